@@ -46,6 +46,7 @@ class LayerCache:
     kv: Optional[KVView]
     state: Optional[torch.Tensor]   # [slots, *shape]
     writable: bool
+    states: Optional[Dict[str, torch.Tensor]] = None    # the call's named states, each [slots, *shape]
 
 
 class KVGroup:
@@ -163,10 +164,14 @@ class SequenceCache:
                 self._group_of[call] = group
 
         self.states: Dict[int, torch.Tensor] = {}
+        self.named_states: Dict[int, Dict[str, torch.Tensor]] = {}
         for call, need in enumerate(needs):
             if need is not None and need.state is not None:
                 self.states[call] = torch.zeros((max_slots, *need.state.shape),
                                                 dtype=need.state.dtype, device=device)
+            if need is not None and need.states:
+                self.named_states[call] = {name: torch.zeros((max_slots, *spec.shape), dtype=spec.dtype, device=device)
+                                           for name, spec in need.states}
 
     # -- slots ---------------------------------------------------------------
     def alloc_slot(self) -> int:
@@ -174,6 +179,9 @@ class SequenceCache:
         self.lengths[slot] = 0
         for state in self.states.values():
             state[slot].zero_()
+        for named in self.named_states.values():
+            for state in named.values():
+                state[slot].zero_()
         return slot
 
     def free_slot(self, slot: int) -> None:
@@ -228,7 +236,7 @@ class SequenceCache:
         self._require(slot)
         if length > self.lengths[slot]:
             raise CacheError(f"slot {slot}: cannot truncate {self.lengths[slot]} tokens to {length}")
-        if self.states and length != self.lengths[slot]:
+        if (self.states or self.named_states) and length != self.lengths[slot]:
             raise CacheError("a cache with per-sequence state cannot be truncated")
         for group in self.groups:
             # a window has let go of the blocks below its floor: a shorter sequence that would look there again cannot be had
@@ -252,7 +260,8 @@ class SequenceCache:
         if group is not None:
             index = group.calls.index(source)
             kv = KVView(group.spec, group.k[index], group.v[index], group.device_table)
-        return LayerCache(kv=kv, state=self.states.get(source), writable=(source == call))
+        return LayerCache(kv=kv, state=self.states.get(source), writable=(source == call),
+                          states=self.named_states.get(source))
 
     # -- accounting ----------------------------------------------------------
     def held_blocks(self) -> int:

@@ -280,12 +280,14 @@ def registered_architectures():
 
 def _ensure_builtin() -> None:
     # The built-in architectures register themselves when their module is imported.
-    from ..models import llama  # noqa: F401
+    from ..models import llama, sozopel  # noqa: F401
 
 
 def parse_config(raw: dict):
     """config.json contents -> the typed configuration of its architecture."""
     architectures = raw.get("architectures")
+    if architectures is None and isinstance(raw.get("architecture"), str):      # some designs name themselves under this key
+        architectures = [raw["architecture"]]
     if not isinstance(architectures, list) or not architectures:
         raise ConfigError("config.json: 'architectures' must be a non-empty list")
     return architecture(architectures[0]).config_class.from_dict(raw)

@@ -82,7 +82,7 @@ __device__ __forceinline__ void merge(Seen<OWNED>& into, const Seen<OWNED>& from
 template <typename T, int G, int OWNED>
 __device__ __forceinline__ void attend_blocks(Seen<OWNED> (&seen)[G], int b_begin, int b_end, int first, int pos, const float* qs, float* ps,
                                               const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-                                              const int* __restrict__ table, int n_blocks, int n_kv_heads, int kv_head, int head_dim,
+                                              const int* __restrict__ table, int n_blocks, int n_kv_heads, int kv_head, int head_dim, int value_dim,
                                               float scale, bool biased, const float (&slopes)[G], bool whole_pieces) {
     const int lane = threadIdx.x % XRT_WAVE;
     for (int b = b_begin; b <= b_end; ++b) {
@@ -91,6 +91,7 @@ __device__ __forceinline__ void attend_blocks(Seen<OWNED> (&seen)[G], int b_begi
         const int j = b * XRT_BLOCK_TOKENS + lane;
         const bool valid = j >= first && j <= pos;
         const long head_base = ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * head_dim;
+        const long value_base = ((long)block * n_kv_heads + kv_head) * XRT_BLOCK_TOKENS * value_dim;
         float s[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) s[g] = -INFINITY;
@@ -147,13 +148,13 @@ __device__ __forceinline__ void attend_blocks(Seen<OWNED> (&seen)[G], int b_begi
 #pragma unroll
         for (int i = 0; i < OWNED; ++i) {
             const int d = lane + i * XRT_WAVE;
-            if (d < head_dim) {
+            if (d < value_dim) {
                 float sum[G];
 #pragma unroll
                 for (int g = 0; g < G; ++g) sum[g] = 0.f;
 #pragma unroll 4
                 for (int j0 = j_begin / 8 * 8; j0 <= j_end; j0 += 8) {   // the dim's values in the order of their tokens
-                    const T* piece = v_cache + head_base + cache_value_offset(d, j0, head_dim);
+                    const T* piece = v_cache + value_base + cache_value_offset(d, j0, value_dim);
                     if (whole_pieces) {
                         float value[8];                         // (what lies beyond the sequence's end is loaded and not used)
                         load_piece(piece, value);
@@ -184,23 +185,23 @@ constexpr int CHUNK_WAVES = 8;
 
 template <typename T, int WAVES, int G, int OWNED>
 __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
-    const T* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads, int head_dim,
+    const T* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads, int head_dim, int value_dim,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
-    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes) {
+    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink) {
     __shared__ float qs[G * OWNED * XRT_WAVE];                 // [G][head_dim]
     __shared__ float ps[WAVES][G * XRT_WAVE];
     // what the wavefronts found in the chunks of a round, for the merge: two sets, used in turn (WAVES > 1)
     __shared__ float round_ml[WAVES > 1 ? 2 : 1][WAVES][G][2];
-    extern __shared__ float round_acc[];                       // [2][WAVES][G][head_dim] where WAVES > 1
+    extern __shared__ float round_acc[];                       // [2][WAVES][G][value_dim] where WAVES > 1
     const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE;
     const int sets = n_heads / G;                              // sets of G heads per token
     const int token = blockIdx.x / sets, head0 = blockIdx.x % sets * G;
     const int kv_head = head0 / (n_heads / n_kv_heads);        // (G divides the group: the set shares its key/value head)
-    T* dst = out + ((long)token * n_heads + head0) * head_dim;
+    T* dst = out + ((long)token * n_heads + head0) * value_dim;
     const int slot = slots[token];
     if (slot < 0) {                                            // the whole workgroup leaves
-        for (int e = threadIdx.x; e < G * head_dim; e += WAVES * XRT_WAVE) dst[e] = from_float<T>(0.f);
+        for (int e = threadIdx.x; e < G * value_dim; e += WAVES * XRT_WAVE) dst[e] = from_float<T>(0.f);
         return;
     }
     const int pos = positions[token];
@@ -227,7 +228,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
 #pragma unroll
             for (int g = 0; g < G; ++g) here[g].clear();
             attend_blocks<T, G, OWNED>(here, max(first_block, chunk * CHUNK_BLOCKS), min(last_block, chunk * CHUNK_BLOCKS + CHUNK_BLOCKS - 1),
-                                       first, pos, qs, ps[0], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, scale,
+                                       first, pos, qs, ps[0], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, value_dim, scale,
                                        biased, slopes, whole_pieces);
 #pragma unroll
             for (int g = 0; g < G; ++g) merge(all[g], here[g]);
@@ -238,32 +239,32 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
         int set = 0;
         for (int round = first_chunk; round <= last_chunk; round += WAVES, set ^= 1) {
             const int chunk = round + wave;
-            float* mine = round_acc + ((long)set * WAVES + wave) * G * head_dim;
+            float* mine = round_acc + ((long)set * WAVES + wave) * G * value_dim;
             if (chunk <= last_chunk) {
                 Seen<OWNED> here[G];
 #pragma unroll
                 for (int g = 0; g < G; ++g) here[g].clear();
                 attend_blocks<T, G, OWNED>(here, max(first_block, chunk * CHUNK_BLOCKS), min(last_block, chunk * CHUNK_BLOCKS + CHUNK_BLOCKS - 1),
-                                           first, pos, qs, ps[wave], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, scale,
+                                           first, pos, qs, ps[wave], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, value_dim, scale,
                                            biased, slopes, whole_pieces);
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
 #pragma unroll
                     for (int i = 0; i < OWNED; ++i)
-                        if (lane + i * XRT_WAVE < head_dim) mine[g * head_dim + lane + i * XRT_WAVE] = here[g].acc[i];
+                        if (lane + i * XRT_WAVE < value_dim) mine[g * value_dim + lane + i * XRT_WAVE] = here[g].acc[i];
                     if (lane == 0) { round_ml[set][wave][g][0] = here[g].m; round_ml[set][wave][g][1] = here[g].l; }
                 }
             }
             __syncthreads();                                   // (a set is written again two rounds on, after the next barrier)
             for (int w = 0; w < WAVES && round + w <= last_chunk; ++w) {
-                const float* theirs = round_acc + ((long)set * WAVES + w) * G * head_dim;
+                const float* theirs = round_acc + ((long)set * WAVES + w) * G * value_dim;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     Seen<OWNED> from;
                     from.m = round_ml[set][w][g][0];
                     from.l = round_ml[set][w][g][1];
 #pragma unroll
-                    for (int i = 0; i < OWNED; ++i) from.acc[i] = lane + i * XRT_WAVE < head_dim ? theirs[g * head_dim + lane + i * XRT_WAVE] : 0.f;
+                    for (int i = 0; i < OWNED; ++i) from.acc[i] = lane + i * XRT_WAVE < value_dim ? theirs[g * value_dim + lane + i * XRT_WAVE] : 0.f;
                     merge(all[g], from);
                 }
             }
@@ -272,38 +273,45 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
     }
 #pragma unroll
     for (int g = 0; g < G; ++g) {
+        if (sink) {                                            // one more key, whose score is 0 and whose value is nothing
+            Seen<OWNED> nothing;
+            nothing.clear();
+            nothing.m = 0.f;
+            nothing.l = 1.f;
+            merge(all[g], nothing);
+        }
         const float inv = all[g].l > 0.f ? 1.0f / all[g].l : 0.f;        // llama.rs:566-571
 #pragma unroll
         for (int i = 0; i < OWNED; ++i) {
             const int d = lane + i * XRT_WAVE;
-            if (d < head_dim) dst[g * head_dim + d] = from_float<T>(all[g].acc[i] * inv);
+            if (d < value_dim) dst[g * value_dim + d] = from_float<T>(all[g].acc[i] * inv);
         }
     }
 }
 
 }  // namespace
 
-int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim,
+int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
-                          int window, const float* distance_slopes, hipStream_t s) {
-    XRT_REQUIRE(head_dim <= MAX_HEAD_DIM, "attention: head_dim %d exceeds %d", head_dim, MAX_HEAD_DIM);
+                          int window, const float* distance_slopes, int sink, hipStream_t s) {
+    XRT_REQUIRE(head_dim <= MAX_HEAD_DIM && value_dim > 0 && value_dim <= MAX_HEAD_DIM, "attention: head sizes %d and %d must be at most %d", head_dim, value_dim, MAX_HEAD_DIM);
     // Query heads of a key/value head that a wavefront takes together: as many of the group as 4, for head sizes up to 128
     // (what a lane then owns of a head fits two registers a head), where that still leaves two workgroups to a compute
     // unit (a decode step of few sequences would rather have the workgroups). Either way a head's arithmetic is the same.
     const int group = n_heads / n_kv_heads;
-    int together = head_dim > 2 * XRT_WAVE ? 1 : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
+    int together = max(head_dim, value_dim) > 2 * XRT_WAVE ? 1 : group % 4 == 0 ? 4 : group % 2 == 0 ? 2 : 1;
     if ((long)tokens * (n_heads / together) < 2L * XRT_COMPUTE_UNITS) together = 1;
     const long items = (long)tokens * (n_heads / together);
     XRT_REQUIRE((long)tokens * n_heads < (1L << 31), "attention: too many (token, head) pairs");
-    const int row_width = (n_heads + 2 * n_kv_heads) * head_dim;
+    const int row_width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim;
     // few (token, head) pairs (a decode step): a workgroup of wavefronts each, which take the chunks of keys side by side
     const bool side_by_side = (long)tokens * n_heads <= 8L * XRT_COMPUTE_UNITS;
-    const size_t round_bytes = (size_t)2 * CHUNK_WAVES * together * head_dim * sizeof(float);
+    const size_t round_bytes = (size_t)2 * CHUNK_WAVES * together * value_dim * sizeof(float);
 #define XRT_GENERIC(T, WAVES_, G_, OWNED_)                                                                                \
     attention_generic_kernel<T, WAVES_, G_, OWNED_><<<(unsigned)items, WAVES_ * XRT_WAVE, WAVES_ > 1 ? round_bytes : 0, s>>>( \
-        (const T*)qkv, row_width, n_heads, n_kv_heads, head_dim, (const T*)k_cache, (const T*)v_cache, block_table,       \
-        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes)
+        (const T*)qkv, row_width, n_heads, n_kv_heads, head_dim, value_dim, (const T*)k_cache, (const T*)v_cache, block_table,       \
+        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink)
 #define XRT_GENERIC_WAVES(T, G_, OWNED_) do { if (side_by_side) XRT_GENERIC(T, CHUNK_WAVES, G_, OWNED_); else XRT_GENERIC(T, 1, G_, OWNED_); } while (0)
 #define XRT_GENERIC_SETS(T)                                                                                               \
     do {                                                                                                                  \

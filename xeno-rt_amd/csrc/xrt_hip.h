@@ -181,6 +181,75 @@ int xrt_sample(const float* logits, int rows, int vocab, int* out, const float* 
                long workspace_bytes, void* stream);
 long xrt_sample_workspace(int rows, int vocab);
 
+// ---- mixing along the sequence with state of fixed size per sequence (csrc/sequence_state.hip) -------------------------
+// A step's sequences are described by seq_offsets [n_seqs + 1] (where each one's tokens begin among the packed tokens) and
+// seq_slots [n_seqs] (negative: padding, whose output rows become zeros); per-sequence state is indexed by slot.
+
+// Causal convolution over time on each channel: out[o][t][c] = sum_j w[o][c][j] * x[t - taps + 1 + j][c] with the inputs
+// before the step taken from state [slots][taps - 1][channels] (float32; zeros at a sequence's start), which afterwards holds
+// the sequence's last taps - 1 inputs. x rows are x_stride elements apart; out is [n_out][tokens][channels] of x's type.
+// XRT_CONV_PLUS_INPUT adds x[t][c]; XRT_CONV_TOWARDS_LAST (taps 2, w [n_out][channels]) gives x + (x[t - 1] - x) * w.
+enum { XRT_CONV_PLAIN = 0, XRT_CONV_PLUS_INPUT = 1, XRT_CONV_TOWARDS_LAST = 2 };
+int xrt_short_conv(const void* x, int dtype, long tokens, long x_stride, int channels, const void* w, int w_dtype, int taps,
+                   int n_out, int mode, float* state, const int* seq_offsets, const int* seq_slots, int n_seqs, int max_count,
+                   void* out, void* stream);
+
+// Per head a state S [dim][vdim] (float32, state [slots][heads][dim][vdim]): with q, k (rows of heads x dim, times q_scale and
+// k_scale) and v (heads x vdim) of every token in turn  S <- diag(decay) S + k v^T  and  o = S^T q;  with a bonus u [heads][dim]
+// the token is read before the update, o = (S + diag(u) k v^T)^T q. The decay of a key channel: decay[head] for all tokens
+// (XRT_DECAY_PER_HEAD), or from decay [tokens][heads * dim] (float32) plus decay_bias [heads * dim] (or null): the number itself
+// (GIVEN), exp(-exp(z)) (EXP_NEG_EXP) or sigmoid(z)^decay_power (SIGMOID_POWER). Then, per head: o / sqrt(mean(o^2) + eps) if
+// norm, times norm_weight ([vdim] for all heads, or [heads * vdim]) if given, times gate (rows of heads x vdim of the element
+// type, through silu with XRT_GATE_SILU) if given; out rows are heads x vdim.
+enum { XRT_DECAY_PER_HEAD = 0, XRT_DECAY_GIVEN = 1, XRT_DECAY_EXP_NEG_EXP = 2, XRT_DECAY_SIGMOID_POWER = 3 };
+enum { XRT_GATE_PLAIN = 0, XRT_GATE_SILU = 1 };
+typedef struct {
+    const void *q, *k, *v;
+    long q_stride, k_stride, v_stride;
+    int heads, dim, vdim;
+    float q_scale, k_scale;
+    int decay_mode;
+    const float* decay;
+    const void* decay_bias;
+    int decay_bias_dtype;
+    float decay_power;
+    const void* bonus;
+    int bonus_dtype;
+    float* state;
+    int norm;
+    float eps;
+    const void* norm_weight;
+    int norm_weight_dtype, norm_weight_per_head;
+    const void* gate;
+    long gate_stride;
+    int gate_act;
+    void* out;
+} xrt_recurrence;
+int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, const int* seq_offsets, const int* seq_slots, int n_seqs, void* stream);
+
+// residual[r] += scale * (x0[r] / rms(x0[r]) * gain0 + x1[r] / rms(x1[r]) * gain1); x float32 [rows][width], x1 may be null
+int xrt_add_normed(float* residual, const float* x0, const void* gain0, const float* x1, const void* gain1, int gain_dtype,
+                   long rows, int width, float eps, float scale, void* stream);
+
+// out[i] = f(x[i]): tanh, silu, or xIELU with params = (p, q): z > 0: softplus(p) z^2 + z / 2, else (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2
+enum { XRT_UNARY_TANH = 0, XRT_UNARY_SILU = 1, XRT_UNARY_XIELU = 2 };
+int xrt_activation(const void* x, int x_dtype, void* out, int out_dtype, long count, int kind, const void* params, int params_dtype,
+                   void* stream);
+
+// out[t] += table[ids[t]] (out float32 [tokens][width]; ids outside the table's rows add nothing)
+int xrt_rows_add(const void* table, int dtype, const int* ids, float* out, long tokens, int width, int rows, void* stream);
+
+// The step's keys (rows of n_kv_heads x head_dim) and values (n_kv_heads x value_dim) into the cache at their tokens' places.
+int xrt_kv_store(const void* k, long k_stride, const void* v, long v_stride, int dtype, long tokens, int n_kv_heads, int head_dim,
+                 int value_dim, const int* positions, const int* slots, void* k_cache, void* v_cache, const int* block_table,
+                 int table_stride, int n_blocks, void* stream);
+
+// The general attention kernel with values of a width of their own and, with sink, one more key of score 0 that has no value.
+int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
+                          const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
+                          const int* positions, const int* slots, void* out, float scale, int window,
+                          const float* distance_slopes, int sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -90,6 +90,9 @@ class Engine:
     def load(cls, folder: str, dtype="bfloat16", **options) -> "Engine":
         """From a folder with config.json and model.safetensors (or shards with an index)."""
         config = load_config(folder)
+        if hasattr(config, "completed_from"):           # a design that leaves some sizes to the tensors' shapes
+            from ..weights import tensor_shapes
+            config = config.completed_from(tensor_shapes(folder))
         spec = architecture(config.architecture).build(config)
         tensors = CheckpointSource(folder, spec.weight_specs(), spec.ignored_names())
         return cls(spec, tensors, dtype=dtype, **options)

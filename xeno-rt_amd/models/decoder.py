@@ -90,7 +90,7 @@ class DecoderModel:
     def forward(self, batch, cache) -> torch.Tensor:
         """Logits [len(batch.logit_rows), vocab] in float32 for the tokens of `batch`."""
         spec = self.spec
-        x = spec.embedding.forward(batch.token_ids)
+        x = spec.embedding.forward(batch.token_ids, batch.positions)
         h = None            # the next block's first norm of x, where the block before it has made it already
         for index, call in enumerate(spec.schedule):
             block = spec.layers[call.layer]

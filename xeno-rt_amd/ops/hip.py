@@ -124,6 +124,23 @@ class _LinearNorm(ctypes.Structure):
                 ("gain_dtype", ctypes.c_int), ("squares_out", ctypes.c_void_p)]
 
 
+class _Recurrence(ctypes.Structure):
+    _fields_ = [("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+                ("q_stride", ctypes.c_long), ("k_stride", ctypes.c_long), ("v_stride", ctypes.c_long),
+                ("heads", ctypes.c_int), ("dim", ctypes.c_int), ("vdim", ctypes.c_int),
+                ("q_scale", ctypes.c_float), ("k_scale", ctypes.c_float), ("decay_mode", ctypes.c_int),
+                ("decay", ctypes.c_void_p), ("decay_bias", ctypes.c_void_p), ("decay_bias_dtype", ctypes.c_int),
+                ("decay_power", ctypes.c_float), ("bonus", ctypes.c_void_p), ("bonus_dtype", ctypes.c_int),
+                ("state", ctypes.c_void_p), ("norm", ctypes.c_int), ("eps", ctypes.c_float),
+                ("norm_weight", ctypes.c_void_p), ("norm_weight_dtype", ctypes.c_int), ("norm_weight_per_head", ctypes.c_int),
+                ("gate", ctypes.c_void_p), ("gate_stride", ctypes.c_long), ("gate_act", ctypes.c_int), ("out", ctypes.c_void_p)]
+
+
+CONV_MODES = {"plain": 0, "plus_input": 1, "towards_last": 2}          # XRT_CONV_* of the library
+DECAY_MODES = {"per_head": 0, "given": 1, "exp_neg_exp": 2, "sigmoid_power": 3}      # XRT_DECAY_*
+UNARY = {"tanh": 0, "silu": 1, "xielu": 2}                             # XRT_UNARY_*
+
+
 class HipOps:
     name = "hip"
     _instance = None
@@ -162,7 +179,9 @@ class HipOps:
         for name in ("xrt_embed", "xrt_add", "xrt_rmsnorm", "xrt_linear", "xrt_qkv_prepare",
                      "xrt_attention", "xrt_sample", "xrt_linear_takes_norm", "xrt_linear_norm_tiles", "xrt_linear_normed", "xrt_linear_qkv", "xrt_random_normal",
                      "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits", "xrt_block_tokens",
-                     "xrt_attention_finishes_qkv", "xrt_attention_finishing", "xrt_rope_table"):
+                     "xrt_attention_finishes_qkv", "xrt_attention_finishing", "xrt_rope_table", "xrt_short_conv",
+                     "xrt_linear_recurrence", "xrt_add_normed", "xrt_activation", "xrt_rows_add", "xrt_kv_store",
+                     "xrt_attention_general"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -405,10 +424,16 @@ class HipOps:
                                             None if norm is None else ctypes.byref(norm), *prepare,
                                             _ptr(workspace), ctypes.c_long(need), self._stream(a)))
 
-    def _kv(self, kv, like, n_kv_heads, head_dim):
+    def _kv(self, kv, like, n_kv_heads, head_dim, value_dim=None):
         from ..cache import BLOCK_TOKENS
         n_blocks = kv.k.shape[0]
         self._require(kv.k, "key cache", like.dtype, (n_blocks, n_kv_heads, BLOCK_TOKENS, head_dim), like)
+        if value_dim is not None:
+            self._require(kv.v, "value cache", like.dtype, (n_blocks, n_kv_heads, value_dim, BLOCK_TOKENS), like)
+            self._require(kv.block_table, "block table", torch.int32, None, like)
+            if kv.block_table.dim() != 2:
+                raise KernelError("block table: expected [slots, blocks]")
+            return kv.k, kv.v, kv.block_table, kv.block_table.shape[1], n_blocks
         if kv.v.dim() == 4 and kv.v.shape[2] != head_dim:
             raise KernelError(f"value cache: values of width {kv.v.shape[2]} beside keys of width {head_dim}: the attention "
                               "kernels of this library take values as wide as the keys (a mixer whose values differ "
@@ -438,13 +463,16 @@ class HipOps:
                                                         0 if rope_table is None else int(rope_table.shape[0]), int(batch.max_context)))
 
     def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None,
-                  finish: Optional[QkvFinish] = None):
+                  finish: Optional[QkvFinish] = None, value_dim: Optional[int] = None, sink: bool = False):
         """Causal attention of the step's tokens over the cache. distance_slopes: float32 [n_heads], or None; a key at
         position j adds slope * (j - P) to the scaled score of the query at position P. finish: what is still to do to
         q, k and v (only where `attention_finishes_qkv` says so); the cache must be writable then."""
         from ..cache import BLOCK_TOKENS
         if finish is not None:
             return self._attention_finishing(qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish)
+        if sink or (value_dim is not None and value_dim != head_dim):
+            return self._attention_general(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, window,
+                                           distance_slopes, sink)
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
         self._require(qkv, "qkv", None, (tokens, width))
@@ -477,6 +505,155 @@ class HipOps:
             _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out),
             ctypes.c_float(scale), int(window or 0), _ptr(distance_slopes), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
+
+    def _attention_general(self, qkv, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window, distance_slopes, sink):
+        """Rows of qkv are [n_heads x head_dim | n_kv_heads x head_dim | n_kv_heads x value_dim], rows of out n_heads x value_dim.
+        sink: the softmax's denominator has one more (a key of score 0 without a value)."""
+        tokens = qkv.shape[0]
+        self._require(qkv, "qkv", None, (tokens, (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim))
+        self._require(out, "attention out", qkv.dtype, (tokens, n_heads * value_dim), qkv)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), qkv)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), qkv)
+        k_cache, v_cache, table, stride, n_blocks = self._kv(kv, qkv, n_kv_heads, head_dim, value_dim)
+        if distance_slopes is not None:
+            self._require(distance_slopes, "attention distance_slopes", torch.float32, (n_heads,), qkv)
+        self._check(self.lib.xrt_attention_general(
+            _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, value_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table), stride,
+            n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale), int(window or 0),
+            _ptr(distance_slopes), int(bool(sink)), self._stream(qkv)))
+
+    # -- mixing along the sequence with state of fixed size ----------------------------
+    def _rows(self, tensor, what, width=None, dtype=None, like=None):
+        """A matrix whose rows are contiguous (it may be some columns of a wider one); returns its row stride."""
+        if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda or tensor.dim() != 2 or (tensor.shape[1] > 1 and tensor.stride(1) != 1):
+            raise KernelError(f"{what}: expected a matrix on the GPU with contiguous rows")
+        if like is not None and (tensor.device != like.device or tensor.shape[0] != like.shape[0]):
+            raise KernelError(f"{what}: {tuple(tensor.shape)} on {tensor.device} does not go with {tuple(like.shape)} on {like.device}")
+        if width is not None and tensor.shape[1] != width:
+            raise KernelError(f"{what}: {tensor.shape[1]} columns, expected {width}")
+        if dtype is not None and tensor.dtype != dtype:
+            raise KernelError(f"{what}: dtype {tensor.dtype}, expected {dtype}")
+        return int(tensor.stride(0)) if tensor.shape[0] > 1 else int(tensor.shape[1])
+
+    def _sequences(self, batch, tokens, like):
+        n = int(batch.n_sequences)
+        self._require(batch.sequence_offsets, "sequence offsets", torch.int32, (n + 1,), like)
+        self._require(batch.sequence_slots, "sequence slots", torch.int32, (n,), like)
+        if int(batch.n_tokens) != tokens:
+            raise KernelError(f"the step has {batch.n_tokens} tokens, the operand {tokens} rows")
+        return _ptr(batch.sequence_offsets), _ptr(batch.sequence_slots), n
+
+    def short_conv(self, x, w, state, batch, out, mode="plain"):
+        """out[o, t, c] = sum_j w[o, c, j] x[t - taps + 1 + j, c] along each sequence; state [slots, taps - 1, channels] (float32)
+        holds what came before the step and is brought up to date. w is [channels, taps] or [n_out, channels, taps]; mode
+        "plus_input" adds x, "towards_last" (w [n_out, channels], two taps) gives x + (x[t - 1] - x) * w."""
+        if mode not in CONV_MODES:
+            raise KernelError(f"short_conv: mode must be one of {sorted(CONV_MODES)}")
+        tokens, channels = x.shape
+        stride = self._rows(x, "short_conv x")
+        if mode == "towards_last":
+            taps, n_out = 2, (1 if w.dim() == 1 else w.shape[0])
+            self._require(w, "short_conv w", None, (channels,) if w.dim() == 1 else (n_out, channels), x)
+        else:
+            taps, n_out = w.shape[-1], (1 if w.dim() == 2 else w.shape[0])
+            self._require(w, "short_conv w", None, (channels, taps) if w.dim() == 2 else (n_out, channels, taps), x)
+        self._require(state, "short_conv state", torch.float32, (state.shape[0], taps - 1, channels), x)
+        self._require(out, "short_conv out", x.dtype, (tokens, channels) if out.dim() == 2 and n_out == 1 else (n_out, tokens, channels), x)
+        offsets, slots, n = self._sequences(batch, tokens, x)
+        self._check(self.lib.xrt_short_conv(_ptr(x), _code(x), ctypes.c_long(tokens), ctypes.c_long(stride), channels, _ptr(w), _code(w), taps,
+                                            n_out, CONV_MODES[mode], _ptr(state), offsets, slots, n, int(batch.max_count), _ptr(out),
+                                            self._stream(x)))
+
+    def linear_recurrence(self, q, k, v, state, batch, out, heads, dim, vdim, decay, decay_mode="per_head", decay_bias=None,
+                          decay_power=1.0, q_scale=1.0, k_scale=1.0, bonus=None, norm_eps=None, norm_weight=None, gate=None,
+                          gate_activation="silu"):
+        """Per sequence and head S <- diag(decay) S + k v^T, o = S^T q (with `bonus` [heads, dim]: o = (S + diag(bonus) k v^T)^T q
+        before the update); state [slots, heads, dim, vdim] float32. decay: float32 [heads] ("per_head") or [tokens, heads * dim]
+        ("given": the decay itself; "exp_neg_exp": exp(-exp(z + bias)); "sigmoid_power": sigmoid(z + bias)^decay_power). Then per head
+        o / sqrt(mean(o^2) + norm_eps) (if norm_eps is given), times norm_weight ([vdim] or [heads * vdim]), times gate
+        (through silu, or "plain")."""
+        tokens = q.shape[0]
+        record = _Recurrence()
+        record.q_stride = self._rows(q, "recurrence q", heads * dim)
+        record.k_stride = self._rows(k, "recurrence k", heads * dim, q.dtype, q)
+        record.v_stride = self._rows(v, "recurrence v", heads * vdim, q.dtype, q)
+        record.q, record.k, record.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+        record.heads, record.dim, record.vdim = heads, dim, vdim
+        record.q_scale, record.k_scale = float(q_scale), float(k_scale)
+        if decay_mode not in DECAY_MODES:
+            raise KernelError(f"linear_recurrence: decay_mode must be one of {sorted(DECAY_MODES)}")
+        record.decay_mode = DECAY_MODES[decay_mode]
+        self._require(decay, "recurrence decay", torch.float32, (heads,) if decay_mode == "per_head" else (tokens, heads * dim), q)
+        record.decay = decay.data_ptr()
+        if decay_bias is not None:
+            self._require(decay_bias, "recurrence decay_bias", None, (heads * dim,), q)
+            record.decay_bias, record.decay_bias_dtype = decay_bias.data_ptr(), _code(decay_bias)
+        record.decay_power = float(decay_power)
+        if bonus is not None:
+            self._require(bonus, "recurrence bonus", None, (heads, dim), q)
+            record.bonus, record.bonus_dtype = bonus.data_ptr(), _code(bonus)
+        self._require(state, "recurrence state", torch.float32, (state.shape[0], heads, dim, vdim), q)
+        record.state = state.data_ptr()
+        record.norm, record.eps = int(norm_eps is not None), float(norm_eps or 0.0)
+        if norm_weight is not None:
+            if tuple(norm_weight.shape) not in ((vdim,), (heads * vdim,)):
+                raise KernelError(f"recurrence norm_weight: shape {tuple(norm_weight.shape)}, expected ({vdim},) or ({heads * vdim},)")
+            self._require(norm_weight, "recurrence norm_weight", None, None, q)
+            record.norm_weight, record.norm_weight_dtype = norm_weight.data_ptr(), _code(norm_weight)
+            record.norm_weight_per_head = int(tuple(norm_weight.shape) == (heads * vdim,) and heads > 1)
+        if gate is not None:
+            record.gate_stride = self._rows(gate, "recurrence gate", heads * vdim, q.dtype, q)
+            record.gate, record.gate_act = gate.data_ptr(), {"plain": 0, "silu": 1}[gate_activation]
+        self._require(out, "recurrence out", q.dtype, (tokens, heads * vdim), q)
+        record.out = out.data_ptr()
+        offsets, slots, n = self._sequences(batch, tokens, q)
+        self._check(self.lib.xrt_linear_recurrence(ctypes.byref(record), _code(q), offsets, slots, n, self._stream(q)))
+
+    def add_normed(self, residual, parts, eps, scale=1.0):
+        """residual += scale * sum over (x, gain) in parts of x / sqrt(mean(x^2) + eps) * gain; x float32 like residual; one or two parts."""
+        self._require(residual, "add_normed residual", torch.float32)
+        if residual.dim() != 2 or not 1 <= len(parts) <= 2:
+            raise KernelError("add_normed: a residual [rows, width] and one or two parts")
+        rows, width = residual.shape
+        for x, gain in parts:
+            self._require(x, "add_normed x", torch.float32, (rows, width), residual)
+            self._require(gain, "add_normed gain", parts[0][1].dtype, (width,), residual)
+        (x0, g0), (x1, g1) = parts[0], (parts[1] if len(parts) == 2 else (None, None))
+        self._check(self.lib.xrt_add_normed(_ptr(residual), _ptr(x0), _ptr(g0), _ptr(x1), _ptr(g1), _code(g0), ctypes.c_long(rows), width,
+                                            ctypes.c_float(eps), ctypes.c_float(scale), self._stream(residual)))
+
+    def activation(self, x, out, kind, params=None):
+        """out = f(x) elementwise in float32: "tanh", "silu", or "xielu" with params = (p, q) on the device."""
+        if kind not in UNARY:
+            raise KernelError(f"activation: kind must be one of {sorted(UNARY)}")
+        self._require(x, "activation x")
+        self._require(out, "activation out", None, x.shape, x)
+        if kind == "xielu":
+            self._require(params, "activation params", None, (2,), x)
+        self._check(self.lib.xrt_activation(_ptr(x), _code(x), _ptr(out), _code(out), ctypes.c_long(x.numel()), UNARY[kind],
+                                            _ptr(params), 0 if params is None else _code(params), self._stream(x)))
+
+    def rows_add(self, table, ids, out):
+        """out[t] += table[ids[t]]; out float32 [tokens, width]."""
+        rows, width = table.shape
+        tokens = ids.shape[0]
+        self._require(table, "rows_add table")
+        self._require(ids, "rows_add ids", torch.int32, (tokens,), table)
+        self._require(out, "rows_add out", torch.float32, (tokens, width), table)
+        self._check(self.lib.xrt_rows_add(_ptr(table), _code(table), _ptr(ids), _ptr(out), ctypes.c_long(tokens), width, rows,
+                                          self._stream(out)))
+
+    def kv_store(self, k, v, n_kv_heads, head_dim, value_dim, kv, batch):
+        """The step's keys k [tokens, n_kv_heads * head_dim] and values v [tokens, n_kv_heads * value_dim] into the cache."""
+        tokens = k.shape[0]
+        k_stride = self._rows(k, "kv_store k", n_kv_heads * head_dim)
+        v_stride = self._rows(v, "kv_store v", n_kv_heads * value_dim, k.dtype, k)
+        k_cache, v_cache, table, stride, n_blocks = self._kv(kv, k, n_kv_heads, head_dim, value_dim)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), k)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), k)
+        self._check(self.lib.xrt_kv_store(_ptr(k), ctypes.c_long(k_stride), _ptr(v), ctypes.c_long(v_stride), _code(k), ctypes.c_long(tokens),
+                                          n_kv_heads, head_dim, value_dim, _ptr(batch.positions), _ptr(batch.slots), _ptr(k_cache),
+                                          _ptr(v_cache), _ptr(table), stride, n_blocks, self._stream(k)))
 
     def _attention_finishing(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish: QkvFinish):
         from ..cache import BLOCK_TOKENS

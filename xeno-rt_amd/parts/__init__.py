@@ -1,15 +1,20 @@
 """Parts that models are built from."""
 from .base import (Block, CacheNeeds, FeedForward, HalfSplitRotation, KVSpec, Mixer, Norm, Part, PositionEncoding,
                    Runtime, StateSpec, WeightSpec, create_part, register_part, registered_parts)
-from .norm import RMSNorm
-from .position import NoPosition, Rotary
+from .norm import RMSNorm, ScalarRMSNorm
+from .position import DistanceSlopes, NoPosition, Rotary
+from .convolution import ShortConvolution, TokenShift
 from .attention import Attention
-from .feedforward import GatedMLP
+from .recurrent import GatedLinearAttention, Retention, TimeMixWKV
+from .parallel import ParallelMixer
+from .feedforward import DenseMLP, GatedMLP
 from .block import PreNormBlock
-from .embedding import Embedding, OutputHead
+from .embedding import Embedding, OutputHead, PositionedEmbedding
 
 __all__ = [
     "Block", "CacheNeeds", "FeedForward", "HalfSplitRotation", "KVSpec", "Mixer", "Norm", "Part", "PositionEncoding",
     "Runtime", "StateSpec", "WeightSpec", "create_part", "register_part", "registered_parts",
     "RMSNorm", "NoPosition", "Rotary", "Attention", "GatedMLP", "PreNormBlock", "Embedding", "OutputHead",
+    "ScalarRMSNorm", "DistanceSlopes", "ShortConvolution", "TokenShift", "GatedLinearAttention", "Retention", "TimeMixWKV",
+    "ParallelMixer", "DenseMLP", "PositionedEmbedding",
 ]

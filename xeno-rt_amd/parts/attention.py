@@ -11,6 +11,13 @@ added to the residual stream.
 Q, K and V are bound as one matrix [(n_heads + 2 n_kv_heads) head_dim][hidden], so
 one product reads the normed activations once (the reference fuses the three
 dispatches, llama.rs:447-464).
+
+Beyond the reference's model, as options: values of a width of their own (`value_dim`), a short causal convolution
+over time on every channel of q, k and v right after the projection (`convolution`, whose last inputs are kept per
+sequence), a softmax with one more in its denominator (`sink`: a key of score 0 that has no value), a window, a
+position encoding that biases the scores by distance, and tensor names of the caller's choice (`names`). With any of
+the first three the step takes the general attention kernel, and the keys and values reach the cache through a
+kernel of their own.
 """
 from __future__ import annotations
 
@@ -27,16 +34,27 @@ class Attention(Mixer):
 
     @property
     def capturable(self) -> bool:
-        return self.position is None or self.position.capturable
+        return ((self.position is None or self.position.capturable)
+                and (getattr(self, "convolution", None) is None or self.convolution.capturable))
 
     def __init__(self, prefix: str, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: Optional[PositionEncoding] = None, qk_norm: bool = False,
                  qk_norm_eps: float = 0.0, scale: Optional[float] = None,
-                 window: Optional[int] = None):
+                 window: Optional[int] = None, value_dim: Optional[int] = None, sink: bool = False,
+                 convolution=None, names: Optional[Dict[str, str]] = None):
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
             raise ValueError(f"head counts {n_heads}/{n_kv_heads}: the first must be a multiple of the second")
-        if head_dim <= 0 or head_dim % 2 != 0:          # llama.rs:125-128 takes any size; the rotation pairs dims, so an even one
+        rotates = position is not None and position.rotation() is not None
+        if head_dim <= 0 or (rotates and head_dim % 2 != 0):          # llama.rs:125-128 takes any size; a rotation pairs dims, so an even one
             raise ValueError(f"head_dim {head_dim} must be positive and even")
+        self.value_dim = head_dim if value_dim is None else int(value_dim)
+        self.sink = bool(sink)
+        self.convolution = convolution
+        self.general = self.sink or self.value_dim != head_dim or convolution is not None
+        if self.general and (qk_norm or rotates):
+            raise ValueError("attention with a sink, a convolution or values of another width takes neither head norms nor a rotation")
+        self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+                      "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", **(names or {})}
         self.prefix = prefix
         self.hidden = hidden
         self.n_heads = n_heads
@@ -49,44 +67,84 @@ class Attention(Mixer):
         self.window = window
         self.q_width = n_heads * head_dim
         self.kv_width = n_kv_heads * head_dim
+        self.v_width = n_kv_heads * self.value_dim
         self.w_qkv = None
         self.w_o = None
         self.q_norm = None
         self.k_norm = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        p = self.prefix
+        p, n = self.prefix, self.names
         specs = {
-            p + "q_proj.weight": WeightSpec((self.q_width, self.hidden)),
-            p + "k_proj.weight": WeightSpec((self.kv_width, self.hidden)),
-            p + "v_proj.weight": WeightSpec((self.kv_width, self.hidden)),
-            p + "o_proj.weight": WeightSpec((self.hidden, self.q_width)),
+            p + n["q"]: WeightSpec((self.q_width, self.hidden)),
+            p + n["k"]: WeightSpec((self.kv_width, self.hidden)),
+            p + n["v"]: WeightSpec((self.v_width, self.hidden)),
+            p + n["o"]: WeightSpec((self.hidden, self.n_heads * self.value_dim)),
         }
         if self.qk_norm:
-            specs[p + "q_norm.weight"] = WeightSpec((self.head_dim,), init="ones", kind="vector")
-            specs[p + "k_norm.weight"] = WeightSpec((self.head_dim,), init="ones", kind="vector")
+            specs[p + n["q_norm"]] = WeightSpec((self.head_dim,), init="ones", kind="vector")
+            specs[p + n["k_norm"]] = WeightSpec((self.head_dim,), init="ones", kind="vector")
+        if self.convolution is not None:
+            specs.update(self.convolution.weight_specs())
         return specs
 
     def cache_needs(self) -> CacheNeeds:
-        return CacheNeeds(kv=KVSpec(self.n_kv_heads, self.head_dim, self.window))
+        needs = CacheNeeds(kv=KVSpec(self.n_kv_heads, self.head_dim, self.window,
+                                     None if self.value_dim == self.head_dim else self.value_dim))
+        return needs if self.convolution is None else needs.merged(self.convolution.cache_needs())
 
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        p = self.prefix
+        p, n = self.prefix, self.names
         if self.position is not None:
             self.position.bind(tensors, runtime)
+        if self.general:
+            if self.convolution is not None:
+                self.convolution.bind(tensors, runtime)
+            self.w_qkv = runtime.weight([tensors[p + n[name]] for name in "qkv"])
+            self.w_o = runtime.weight(tensors[p + n["o"]])
+            return
         # q and k heads that a rotation over the whole head turns: their pairs are kept side by side
         rotation = None if self.position is None else self.position.rotation()
         whole = rotation is not None and rotation.rope_dim == self.head_dim
-        self.w_qkv = runtime.weight([tensors[p + name] for name in ("q_proj.weight", "k_proj.weight", "v_proj.weight")],
+        self.w_qkv = runtime.weight([tensors[p + n[name]] for name in "qkv"],
                                     "rotary", head_dim=self.head_dim,
                                     rotated_heads=self.n_heads + self.n_kv_heads if whole else 0)
-        self.w_o = runtime.weight(tensors[p + "o_proj.weight"])
+        self.w_o = runtime.weight(tensors[p + n["o"]])
         if self.qk_norm:
-            self.q_norm = runtime.vector(tensors[p + "q_norm.weight"])
-            self.k_norm = runtime.vector(tensors[p + "k_norm.weight"])
+            self.q_norm = runtime.vector(tensors[p + n["q_norm"]])
+            self.k_norm = runtime.vector(tensors[p + n["k_norm"]])
+
+    def _attend_general(self, h, batch, cache):
+        """The heads' outputs [tokens, n_heads * value_dim] on the general path: projection, convolution over time, the keys and
+        values into the cache, attention."""
+        rt = self.runtime
+        ops = rt.ops
+        tokens = h.shape[0]
+        qkv = rt.empty((tokens, self.q_width + self.kv_width + self.v_width))
+        ops.linear(h, self.w_qkv, qkv)
+        if self.convolution is not None:
+            qkv = self.convolution.forward(qkv, batch, cache)
+        if cache.writable:
+            ops.kv_store(qkv[:, self.q_width:self.q_width + self.kv_width], qkv[:, self.q_width + self.kv_width:],
+                         self.n_kv_heads, self.head_dim, self.value_dim, cache.kv, batch)
+        slopes = None if self.position is None else self.position.score_slopes()
+        out = rt.empty((tokens, self.n_heads * self.value_dim))
+        ops.attention(qkv, self.n_heads, self.n_kv_heads, self.head_dim, cache.kv, batch, out, scale=self.scale, window=self.window,
+                      distance_slopes=slopes, value_dim=self.value_dim, sink=self.sink)
+        return out
+
+    def forward_into(self, h, batch, cache, out: torch.Tensor) -> None:
+        """The mixer's output into `out` (float32 [tokens, hidden]) instead of onto the residual stream: for an attention
+        that is one of several mixers side by side."""
+        if not self.general:
+            raise NotImplementedError("only the general path writes its output aside")
+        self.runtime.ops.linear(self._attend_general(h, batch, cache), self.w_o, out)
 
     def forward(self, h, batch, cache, residual: torch.Tensor, then=None):
+        if self.general:
+            self.runtime.ops.linear(self._attend_general(h, batch, cache), self.w_o, residual, accumulate=True)
+            return None
         rt = self.runtime
         ops = rt.ops
         tokens = h.shape[0]

@@ -61,8 +61,31 @@ class StateSpec:
 
 @dataclass(frozen=True)
 class CacheNeeds:
+    """What one layer call keeps for every sequence: keys and values per token, one state of fixed size, and any
+    number of further states by name (a layer whose parts each keep something: the inputs of a short convolution,
+    the token before, the matrix of a recurrence); `LayerCache.states[name]` is [slots, *shape]."""
     kv: Optional[KVSpec] = None
     state: Optional[StateSpec] = None
+    states: Tuple[Tuple[str, StateSpec], ...] = ()
+
+    def merged(self, *others: "CacheNeeds") -> "CacheNeeds":
+        """This and the others' needs together; at most one of them may keep keys and values, or the unnamed state,
+        and no name may come twice."""
+        kv, state, states = self.kv, self.state, list(self.states)
+        for other in others:
+            if other.kv is not None:
+                if kv is not None:
+                    raise ValueError("two parts of one layer call keep keys and values")
+                kv = other.kv
+            if other.state is not None:
+                if state is not None:
+                    raise ValueError("two parts of one layer call keep an unnamed state")
+                state = other.state
+            states.extend(other.states)
+        names = [name for name, _ in states]
+        if len(set(names)) != len(names):
+            raise ValueError(f"a state's name comes twice in one layer call: {names}")
+        return CacheNeeds(kv, state, tuple(states))
 
 
 class StepArena:

@@ -3,6 +3,10 @@
 The order of the reference's layer loop (crates/xrt-models/src/llama.rs:433-602):
 norm, attention, add, norm, feed-forward, add. The residual stream x is float32
 and is updated in place; each part adds its own output to it.
+
+Options beyond the reference's layer: a block without a feed-forward (only the first sublayer), and an input
+transform per sublayer, a part that is applied to the normed rows before the mixer or the feed-forward reads them
+(`forward(h, batch, cache)`; a short convolution over time, for one) and may keep state in the block's cache entry.
 """
 from __future__ import annotations
 
@@ -12,14 +16,19 @@ from .base import Block, CacheNeeds, Runtime, WeightSpec, register_part
 
 
 class PreNormBlock(Block):
-    def __init__(self, mixer_norm, mixer, feed_forward_norm, feed_forward):
+    def __init__(self, mixer_norm, mixer, feed_forward_norm=None, feed_forward=None, mixer_input=None, feed_forward_input=None):
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.mixer_norm = mixer_norm
         self.mixer = mixer
         self.feed_forward_norm = feed_forward_norm
         self.feed_forward = feed_forward
+        self.mixer_input = mixer_input
+        self.feed_forward_input = feed_forward_input if feed_forward is not None else None
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)
+        return tuple(part for part in (self.mixer_norm, self.mixer_input, self.mixer, self.feed_forward_norm,
+                                       self.feed_forward_input, self.feed_forward) if part is not None)
 
     @property
     def capturable(self) -> bool:
@@ -32,7 +41,8 @@ class PreNormBlock(Block):
         return specs
 
     def cache_needs(self) -> CacheNeeds:
-        return self.mixer.cache_needs()
+        return self.mixer.cache_needs().merged(*[part.cache_needs() for part in (self.mixer_input, self.feed_forward_input)
+                                                 if part is not None])
 
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
@@ -41,12 +51,24 @@ class PreNormBlock(Block):
 
     @property
     def passes_norms(self) -> bool:
-        return bool(getattr(self.mixer, "passes_norms", False))
+        plain = self.mixer_input is None and self.feed_forward_input is None and self.feed_forward is not None
+        return plain and bool(getattr(self.mixer, "passes_norms", False))
 
     def first_norm(self):
         return self.mixer_norm
 
     def forward(self, x, batch, cache, h=None, then=None):
+        if not self.passes_norms:
+            h = self.mixer_norm.forward(x)
+            if self.mixer_input is not None:
+                h = self.mixer_input.forward(h, batch, cache)
+            self.mixer.forward(h, batch, cache, x)
+            if self.feed_forward is not None:
+                h = self.feed_forward_norm.forward(x)
+                if self.feed_forward_input is not None:
+                    h = self.feed_forward_input.forward(h, batch, cache)
+                self.feed_forward.forward(h, batch, x)
+            return None
         if h is None:
             h = self.mixer_norm.forward(x)
         # a norm is left to the products around it only if the part after it reads nothing but products of it

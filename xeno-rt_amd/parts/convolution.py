@@ -1,0 +1,70 @@
+"""Short causal convolutions over time, one filter per channel, and the interpolation of a token with the one before it.
+
+Both look a few tokens back along the sequence, so a sequence keeps its last inputs as state: [taps - 1, channels]
+float32 for every sequence, zeros when it starts. The arithmetic is float32; the result has the compute dtype.
+"""
+from __future__ import annotations
+
+from typing import Dict, Sequence, Tuple
+
+import torch
+
+from .base import CacheNeeds, Part, Runtime, StateSpec, WeightSpec
+
+
+class ShortConvolution(Part):
+    """y[t] = sum_j w[:, j] * u[t - taps + 1 + j] on every channel, zeros before the sequence's start; with
+    plus_input the result is u + y. `names` are the filters' tensors ([channels_i, taps] each), side by side along
+    the channels in the order given (so one pass serves the q, k and v of an attention)."""
+    capturable = True
+
+    def __init__(self, names: Sequence[str], channels: Sequence[int], taps: int, state_name: str, plus_input: bool = False):
+        if taps < 2:
+            raise ValueError(f"a convolution over time needs at least two taps, found {taps}")
+        self.names, self.channel_counts = list(names), [int(c) for c in channels]
+        self.channels = sum(self.channel_counts)
+        self.taps = int(taps)
+        self.state_name = state_name
+        self.plus_input = plus_input
+        self.weight = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {name: WeightSpec((count, self.taps), kind="vector") for name, count in zip(self.names, self.channel_counts)}
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds(states=((self.state_name, StateSpec((self.taps - 1, self.channels))),))
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.weight = torch.cat([runtime.vector(tensors[name]) for name in self.names]).contiguous()
+
+    def forward(self, u: torch.Tensor, batch, cache) -> torch.Tensor:
+        out = self.runtime.empty((u.shape[0], self.channels), u.dtype)
+        self.runtime.ops.short_conv(u, self.weight, cache.states[self.state_name], batch, out,
+                                    mode="plus_input" if self.plus_input else "plain")
+        return out
+
+
+class TokenShift(Part):
+    """For each of several readers its own mix of a token and the one before it: u + (u[t - 1] - u) * mu, with
+    mu [channels] per reader and zeros before the sequence's start. Returns [readers, tokens, channels]."""
+    capturable = True
+
+    def __init__(self, names: Sequence[str], channels: int, state_name: str):
+        self.names, self.channels, self.state_name = list(names), int(channels), state_name
+        self.weight = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {name: WeightSpec((self.channels,), init="zeros", kind="vector") for name in self.names}
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds(states=((self.state_name, StateSpec((1, self.channels))),))
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.weight = torch.stack([runtime.vector(tensors[name]) for name in self.names]).contiguous()
+
+    def forward(self, u: torch.Tensor, batch, cache) -> torch.Tensor:
+        out = self.runtime.empty((len(self.names), u.shape[0], self.channels), u.dtype)
+        self.runtime.ops.short_conv(u, self.weight, cache.states[self.state_name], batch, out, mode="towards_last")
+        return out

@@ -16,34 +16,64 @@ from .base import Part, Runtime, WeightSpec
 class Embedding(Part):
     capturable = True
 
-    def __init__(self, prefix: str, vocab: int, hidden: int):
+    def __init__(self, prefix: str, vocab: int, hidden: int, name: Optional[str] = None):
         self.prefix = prefix
+        self.name = name if name is not None else prefix + "weight"       # the table's tensor
         self.vocab = vocab
         self.hidden = hidden
         self.table = None
         self.shared_with_head = False       # set by an OutputHead that is tied to this table
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {self.prefix + "weight": WeightSpec((self.vocab, self.hidden))}
+        return {self.name: WeightSpec((self.vocab, self.hidden))}
 
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         # a table that is also the head's weight is kept as products like it; one that is only looked up stays plain
-        tensor = tensors[self.prefix + "weight"]
+        tensor = tensors[self.name]
         self.table = runtime.weight(tensor) if self.shared_with_head else runtime.matrix(tensor)
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        """float32 residual stream [tokens, hidden] for int32 token ids."""
+    def forward(self, token_ids: torch.Tensor, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """float32 residual stream [tokens, hidden] for int32 token ids (an embedding that knows nothing of positions
+        does not look at them)."""
         x = self.runtime.empty((token_ids.shape[0], self.hidden), torch.float32)
         self.runtime.ops.embed(self.table, token_ids, x)
+        return x
+
+
+class PositionedEmbedding(Embedding):
+    """x = E[token] + P[position]: a learnt vector for every position from 0 to max_positions - 1, added unscaled."""
+
+    def __init__(self, prefix: str, vocab: int, hidden: int, max_positions: int, name: Optional[str] = None,
+                 positions_name: Optional[str] = None):
+        super().__init__(prefix, vocab, hidden, name)
+        self.max_positions = int(max_positions)
+        self.positions_name = positions_name if positions_name is not None else prefix + "positions"
+        self.position_table = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        specs = super().weight_specs()
+        specs[self.positions_name] = WeightSpec((self.max_positions, self.hidden))
+        return specs
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        self.position_table = runtime.matrix(tensors[self.positions_name])
+
+    def forward(self, token_ids: torch.Tensor, positions: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if positions is None:
+            raise ValueError("an embedding with learnt positions needs the tokens' positions")
+        x = super().forward(token_ids)
+        self.runtime.ops.rows_add(self.position_table, positions, x)
         return x
 
 
 class OutputHead(Part):
     capturable = True
 
-    def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: Optional[Embedding] = None):
+    def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: Optional[Embedding] = None, name: Optional[str] = None):
         self.prefix = prefix
+        self.name = name if name is not None else prefix + "weight"
         self.vocab = vocab
         self.hidden = hidden
         self.tied_to = tied_to
@@ -54,18 +84,18 @@ class OutputHead(Part):
     def weight_specs(self) -> Dict[str, WeightSpec]:
         if self.tied_to is not None:
             return {}
-        return {self.prefix + "weight": WeightSpec((self.vocab, self.hidden))}
+        return {self.name: WeightSpec((self.vocab, self.hidden))}
 
     def ignored_names(self):
         """Tensors that a checkpoint may carry and that this part does not read."""
-        return [self.prefix + "weight"] if self.tied_to is not None else []
+        return [self.name] if self.tied_to is not None else []
 
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
         if self.tied_to is not None:
             self.weight = self.tied_to.table        # the same buffer, not a copy
         else:
-            self.weight = runtime.weight(tensors[self.prefix + "weight"])
+            self.weight = runtime.weight(tensors[self.name])
 
     def forward(self, y: torch.Tensor) -> torch.Tensor:
         logits = self.runtime.empty((y.shape[0], self.vocab), torch.float32, outlives_the_step=True)

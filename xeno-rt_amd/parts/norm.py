@@ -38,4 +38,21 @@ class RMSNorm(Norm):
         return out
 
 
+class ScalarRMSNorm(RMSNorm):
+    """RMSNorm whose gain is one number for all coordinates: y = x / sqrt(mean(x^2) + eps) * g. `name` is the tensor
+    that holds g (shape []); it is spread over the row when bound, and the norm then runs as any other."""
+
+    def __init__(self, name: str, dim: int, eps: float):
+        super().__init__(name, dim, eps)
+        self.name = name
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {self.name: WeightSpec((), init="ones", kind="vector")}
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        Norm.bind(self, tensors, runtime)
+        self.weight = runtime.vector(tensors[self.name]).reshape(1).expand(self.dim).contiguous()
+
+
 register_part("norm", "rmsnorm", RMSNorm)
+register_part("norm", "scalar_rmsnorm", ScalarRMSNorm)

@@ -57,5 +57,27 @@ class NoPosition(PositionEncoding):
         return None
 
 
+class DistanceSlopes(PositionEncoding):
+    """Positions enter the scores only: a key at distance d behind the query loses slope_h * d, with
+    slope_h = 2^(-span (h + 1) / n_heads) for head h. Queries and keys stay as they are."""
+    capturable = True
+
+    def __init__(self, n_heads: int, span: float = 8.0):
+        self.n_heads, self.span = int(n_heads), float(span)
+        self.slopes = None
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        exponents = torch.arange(1, self.n_heads + 1, dtype=torch.float64) * (-self.span / self.n_heads)
+        self.slopes = torch.pow(torch.tensor(2.0, dtype=torch.float64), exponents).to(torch.float32).to(runtime.device)
+
+    def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch) -> None:
+        return None
+
+    def score_slopes(self):
+        return self.slopes
+
+
+register_part("position", "distance_slopes", DistanceSlopes)
 register_part("position", "rotary", Rotary)
 register_part("position", "none", NoPosition)

@@ -180,6 +180,15 @@ class CheckpointSource:
     close = release
 
 
+def tensor_shapes(folder: str) -> Dict[str, tuple]:
+    """name -> shape of every tensor of the folder's checkpoint, from the files' headers alone."""
+    files = CheckpointFiles(folder)
+    try:
+        return {name: tuple(file.entries[name].shape) for name, file in files.where.items()}
+    finally:
+        files.close()
+
+
 def load_tensors(folder: str, expected: Dict[str, WeightSpec], ignored: Iterable[str] = (),
                  device="cpu") -> Dict[str, torch.Tensor]:
     """All expected tensors of `folder` on `device`, after the whole set has been checked."""
