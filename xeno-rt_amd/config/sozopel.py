@@ -46,8 +46,6 @@ def _check_mixer(kind: str, mixer: dict, where: str) -> None:
         _sizes(left, ("heads", "kv_heads", "dim", "vdim", "conv"), where + ".left")
         if left["heads"] % left["kv_heads"] != 0:
             raise ConfigError(f"config.json: {where}.left: {left['heads']} heads cannot share {left['kv_heads']} key/value heads")
-        if left["conv"] < 2:
-            raise ConfigError(f"config.json: {where}.left: 'conv' must be at least 2 taps")
         _number(left, "scale", where + ".left")
         if not isinstance(left.get("mask"), dict):
             raise ConfigError(f"config.json: {where}.left: 'mask' must give the window's size")
@@ -112,8 +110,6 @@ class SozopelConfig:
         if not isinstance(norm, dict) or not isinstance(canon, dict):
             raise ConfigError("config.json: 'norm' and 'canon' must be objects")
         taps = _positive_int(canon, "taps")
-        if taps < 2:
-            raise ConfigError("config.json: canon.taps must be at least 2")
         eos = raw.get("eos_token_id")
         eos = () if eos is None else tuple(eos) if isinstance(eos, list) else (eos,)
         return cls(architecture=str(raw.get("architecture") or raw["architectures"][0]), vocab=_positive_int(raw, "vocab"),

@@ -107,11 +107,11 @@ __global__ void __launch_bounds__(CONV_THREADS) short_conv_kernel(
 
 // ---- linear recurrence -----------------------------------------------------------------------------------------
 
-constexpr int REC_CHUNK = 16;             // tokens whose q, k and decays are staged in LDS at a time
+constexpr int REC_CHUNK = 16;             // tokens whose q, k and decays are staged in LDS at a time (fewer where heads are large)
 
 template <int DIM, bool BONUS, int THREADS>
 __global__ void __launch_bounds__(THREADS) recurrence_kernel(const xrt_recurrence a, int dtype, const int* __restrict__ seq_offsets,
-                                                             const int* __restrict__ seq_slots) {
+                                                             const int* __restrict__ seq_slots, int chunk) {
     extern __shared__ float lds[];
     constexpr int ARRAYS = BONUS ? 4 : 3;                  // q, k, decay and, with a bonus, bonus * k
     const int seq = blockIdx.x, head = blockIdx.y, j = threadIdx.x;
@@ -124,15 +124,15 @@ __global__ void __launch_bounds__(THREADS) recurrence_kernel(const xrt_recurrenc
             for (int c = j; c < vdim; c += blockDim.x) store_from_float(a.out, dtype, t * out_width + (long)head * vdim + c, 0.f);
         return;
     }
-    float* staged = lds;                                   // [REC_CHUNK][ARRAYS][dim]
-    float* raw = lds + REC_CHUNK * ARRAYS * dim;           // [REC_CHUNK][vdim]
+    float* staged = lds;                                   // [chunk][ARRAYS][dim]
+    float* raw = lds + chunk * ARRAYS * dim;               // [chunk][vdim]
     const bool owner = j < vdim;
     float* kept = a.state + (((long)slot * heads + head) * dim) * vdim + j;
     float S[DIM];
 #pragma unroll
     for (int i = 0; i < DIM; ++i) S[i] = owner && i < dim ? kept[(long)i * vdim] : 0.f;
-    for (int t0 = begin; t0 < end; t0 += REC_CHUNK) {
-        const int n = min(REC_CHUNK, end - t0);
+    for (int t0 = begin; t0 < end; t0 += chunk) {
+        const int n = min(chunk, end - t0);
         __syncthreads();                                   // the chunk before is read to its end
         for (int e = threadIdx.x; e < n * dim; e += blockDim.x) {
             const int tt = e / dim, i = e % dim;
@@ -286,8 +286,8 @@ extern "C" int xrt_short_conv(const void* x, int dtype, long tokens, long x_stri
                               void* out, void* stream) {
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "short_conv: unknown dtype %d", dtype);
     XRT_REQUIRE(w_dtype == XRT_F32 || w_dtype == XRT_BF16, "short_conv: unknown weight dtype %d", w_dtype);
-    XRT_REQUIRE(x && w && state && seq_offsets && seq_slots && out, "short_conv: null operand");
-    XRT_REQUIRE(taps >= 2 && taps <= CONV_MAX_TAPS, "short_conv: %d taps, 2 to %d are served", taps, CONV_MAX_TAPS);
+    XRT_REQUIRE(x && w && (state || taps == 1) && seq_offsets && seq_slots && out, "short_conv: null operand");
+    XRT_REQUIRE(taps >= 1 && taps <= CONV_MAX_TAPS, "short_conv: %d taps, 1 to %d are served", taps, CONV_MAX_TAPS);
     XRT_REQUIRE(mode == XRT_CONV_PLAIN || mode == XRT_CONV_PLUS_INPUT || (mode == XRT_CONV_TOWARDS_LAST && taps == 2),
                 "short_conv: unknown mode %d (the interpolation towards the input before has two taps)", mode);
     XRT_REQUIRE(channels > 0 && n_out > 0 && x_stride >= channels && tokens >= 0 && n_seqs >= 0 && max_count >= 0, "short_conv: bad sizes");
@@ -299,8 +299,8 @@ extern "C" int xrt_short_conv(const void* x, int dtype, long tokens, long x_stri
 #define XRT_CONV(T, segments_, phase_)                                                                                     \
     short_conv_kernel<T><<<dim3(n_seqs, segments_, chunks), CONV_THREADS, 0, s>>>((const T*)x, x_stride, channels, w, w_dtype, taps, \
         n_out, mode, state, seq_offsets, seq_slots, (T*)out, tokens, phase_)
-    if (segments == 1) {
-        if (dtype == XRT_F32) XRT_CONV(float, 1, 1); else XRT_CONV(bf16, 1, 1);
+    if (segments == 1 || taps == 1) {                      // (one tap: no state, nothing that one workgroup writes and another reads)
+        if (dtype == XRT_F32) XRT_CONV(float, segments, 1); else XRT_CONV(bf16, segments, 1);
     } else {
         if (dtype == XRT_F32) XRT_CONV(float, segments, 0); else XRT_CONV(bf16, segments, 0);
         if (dtype == XRT_F32) XRT_CONV(float, 1, 2); else XRT_CONV(bf16, 1, 2);
@@ -326,9 +326,10 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
     hipStream_t s = (hipStream_t)stream;
     const bool bonus = a.bonus != nullptr;
     const int threads = (a.vdim + XRT_WAVE - 1) / XRT_WAVE * XRT_WAVE;
-    const size_t lds = (size_t)REC_CHUNK * ((bonus ? 4 : 3) * a.dim + a.vdim) * sizeof(float);
-    XRT_REQUIRE(lds <= 64 * 1024, "linear_recurrence: heads of %d x %d need more LDS than a workgroup has", a.dim, a.vdim);
-#define XRT_REC(DIM_, BONUS_, THREADS_) recurrence_kernel<DIM_, BONUS_, THREADS_><<<dim3(n_seqs, a.heads), threads, lds, s>>>(a, dtype, seq_offsets, seq_slots)
+    const size_t per_token = (size_t)((bonus ? 4 : 3) * a.dim + a.vdim) * sizeof(float);
+    const int chunk = (int)min((size_t)REC_CHUNK, (size_t)(64 * 1024) / per_token);           // (at least 5 with the largest heads)
+    const size_t lds = chunk * per_token;
+#define XRT_REC(DIM_, BONUS_, THREADS_) recurrence_kernel<DIM_, BONUS_, THREADS_><<<dim3(n_seqs, a.heads), threads, lds, s>>>(a, dtype, seq_offsets, seq_slots, chunk)
     // (a workgroup of few wavefronts may keep a whole column of a large state in registers)
 #define XRT_REC_THREADS(DIM_, BONUS_)                                                            \
     do {                                                                                         \

@@ -19,8 +19,8 @@ class ShortConvolution(Part):
     capturable = True
 
     def __init__(self, names: Sequence[str], channels: Sequence[int], taps: int, state_name: str, plus_input: bool = False):
-        if taps < 2:
-            raise ValueError(f"a convolution over time needs at least two taps, found {taps}")
+        if taps < 1:
+            raise ValueError(f"a convolution over time needs at least one tap, found {taps}")
         self.names, self.channel_counts = list(names), [int(c) for c in channels]
         self.channels = sum(self.channel_counts)
         self.taps = int(taps)
@@ -55,7 +55,7 @@ class TokenShift(Part):
         self.weight = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {name: WeightSpec((self.channels,), init="zeros", kind="vector") for name in self.names}
+        return {name: WeightSpec((self.channels,), kind="vector") for name in self.names}
 
     def cache_needs(self) -> CacheNeeds:
         return CacheNeeds(states=((self.state_name, StateSpec((1, self.channels))),))

@@ -76,7 +76,7 @@ class DenseMLP(FeedForward):
         specs = {self.up_name: WeightSpec((self.intermediate, self.hidden)),
                  self.down_name: WeightSpec((self.hidden, self.intermediate))}
         if self.act_name is not None:
-            specs[self.act_name] = WeightSpec((2,), init="zeros", kind="vector")
+            specs[self.act_name] = WeightSpec((2,), kind="vector")
         return specs
 
     def bind(self, tensors, runtime: Runtime) -> None:

@@ -84,7 +84,7 @@ class GatedLinearAttention(_RecurrentMixer):
         return {p + "q": WeightSpec((kd, w)), p + "k": WeightSpec((kd, w)), p + "v": WeightSpec((vd, w)),
                 p + "g": WeightSpec((vd, w)), p + "o": WeightSpec((w, vd)),
                 p + "a1": WeightSpec((self.low_rank, w)), p + "a2": WeightSpec((kd, self.low_rank)),
-                p + "a2.b": WeightSpec((kd,), init="zeros", kind="vector"),
+                p + "a2.b": WeightSpec((kd,), kind="vector"),
                 p + "norm": WeightSpec((self.vdim,), init="ones", kind="vector")}
 
     def cache_needs(self) -> CacheNeeds:
@@ -133,8 +133,8 @@ class TimeMixWKV(_RecurrentMixer):
         p, w, kd = self.prefix, self.hidden, self.heads * self.dim
         specs = {p + name: WeightSpec((kd, w)) for name in "rkvg"}
         specs.update({p + "w1": WeightSpec((self.low_rank, w)), p + "w2": WeightSpec((kd, self.low_rank)),
-                      p + "w0": WeightSpec((kd,), init="zeros", kind="vector"),
-                      p + "u": WeightSpec((self.heads, self.dim), init="zeros", kind="vector"),
+                      p + "w0": WeightSpec((kd,), kind="vector"),
+                      p + "u": WeightSpec((self.heads, self.dim), kind="vector"),
                       p + "norm": WeightSpec((kd,), init="ones", kind="vector"), p + "o": WeightSpec((w, kd))})
         specs.update(self.shift.weight_specs())
         return specs
