@@ -17,6 +17,13 @@ steps end at the context length (4096). Beside the headline the record holds
   * `check`: the logits of one more decode step, run as the recorded graph and again directly (kernels
     launched one by one, no padding of batch or context), compared outside the timed region.
 One JSON line goes to standard output; with more than one GPU asked for it says so and exits with 2.
+
+    python bench.py --design sozopel [--size small|medium|large] [--layers N]
+
+measures instead the Sozopel decoder (layers of time mixing, of windowed attention beside gated linear attention, and of
+retention, in turn) at layer sizes of real models, beside the Llama decoder of the same width, depth, heads and
+feed-forward width: a prefill of 2048 tokens and decode steps at batch 1, 8 and 64 after 1024 tokens of context, each as
+tokens a second and ms; one JSON line with both models' numbers.
 """
 import argparse
 import json
@@ -81,6 +88,70 @@ def prefill_flops(config, lengths):
 
 def sync():
     torch.cuda.synchronize()
+
+
+# ---- the Sozopel design beside the Llama decoder of equal sizes --------------------------------------------------------
+
+DESIGN_SIZES = {        # width, head size, feed-forward width, vocabulary
+    "small": dict(width=1024, head=64, ff=4096, vocab=32000),
+    "medium": dict(width=2048, head=128, ff=8192, vocab=32000),
+    "large": dict(width=4096, head=128, ff=14336, vocab=32000),
+}
+DESIGN_CONTEXT = 1024
+DESIGN_BATCHES = (1, 8, 64)
+
+
+def sozopel_config(size, layers, max_positions):
+    w, d, ff = size["width"], size["head"], size["ff"]
+    heads = w // d
+    kinds = {
+        "wkv": {"type": "wkv", "mlp": None, "mixer": {"heads": heads, "dim": d, "rank": 64}},
+        "parallel": {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
+                     "mixer": {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": d, "vdim": d, "conv": 4,
+                                        "mask": {"size": 512}, "scale": d ** -0.5},
+                               "right": {"heads": max(1, heads // 2), "dim": d, "vdim": 2 * d, "tau": 16.0, "rank": 16}}},
+        "retention": {"type": "retention", "mlp": None,
+                      "mixer": {"heads": max(1, heads // 2), "dim": d, "vdim": 2 * d,
+                                "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(max(1, heads // 2))]}},
+    }
+    order = ("wkv", "parallel", "retention")
+    return {"architecture": "Sozopel", "vocab": size["vocab"], "width": w, "max_positions": max_positions, "norm": {"eps": 1e-6},
+            "canon": {"taps": 4}, "layers": [kinds[order[i % 3]] for i in range(layers)]}
+
+
+def llama_config(size, layers, max_positions):
+    w, d = size["width"], size["head"]
+    return dict(COMMON, architectures=["LlamaForCausalLM"], vocab_size=size["vocab"], hidden_size=w, head_dim=d,
+                num_attention_heads=w // d, num_key_value_heads=max(1, w // d // 4), intermediate_size=size["ff"],
+                num_hidden_layers=layers, rms_norm_eps=1e-6, rope_theta=500000.0, max_position_embeddings=max_positions)
+
+
+def run_design(args) -> int:
+    from xeno_rt_amd.config import parse_config
+    from xeno_rt_amd.engine import Engine
+    size = DESIGN_SIZES[args.size]
+    layers = args.layers if args.layers is not None else 6
+    context = DESIGN_CONTEXT
+    most = max(DESIGN_BATCHES)
+    record = {"design": "sozopel", "beside": "llama", "size": args.size, **size, "layers": layers, "dtype": args.dtype,
+              "context": context, "prefill_tokens": PREFILL_TOKENS, "data": "synthetic token ids, random weights N(0, 0.02)"}
+    for name, raw in (("sozopel", sozopel_config(size, layers, 4096)), ("llama", llama_config(size, layers, 4096))):
+        engine = Engine.random(parse_config(raw), seed=args.seed, dtype=args.dtype, max_tokens=max(most * context, PREFILL_TOKENS),
+                               max_slots=most, max_context=max(context, PREFILL_TOKENS))
+        bench = Bench(engine, args.seed)
+        numbers = {}
+        if args.phase in ("all", "prefill"):
+            seconds = bench.prefill([PREFILL_TOKENS])
+            numbers["prefill_ms"], numbers["prefill_tokens_per_s"] = round(seconds * 1e3, 3), round(PREFILL_TOKENS / seconds, 1)
+        if args.phase in ("all", "decode"):
+            for batch in DESIGN_BATCHES if args.batch is None else (args.batch,):
+                value, ms, _ = bench.decode(batch, args.steps, args.warmup, context)
+                numbers[f"decode_b{batch}_ms"], numbers[f"decode_b{batch}_tokens_per_s"] = round(ms, 4), round(value, 1)
+        record[name] = numbers
+        del bench, engine
+        torch.cuda.empty_cache()
+    print(json.dumps(record), flush=True)
+    return 0
 
 
 def measured_ceilings(ops, device):
@@ -231,12 +302,17 @@ def main() -> int:
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                         help="for profiling: run only the decode steps, or only the prefill (prints a partial record)")
+    parser.add_argument("--design", default=None, choices=["sozopel"],
+                        help="measure this design beside the Llama decoder of equal sizes instead (see the top of this file)")
+    parser.add_argument("--size", default="medium", choices=sorted(DESIGN_SIZES), help="with --design: the layers' sizes")
     parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                         help="with --phase prefill: the prompt's length (the record's prefill is always of 2048 tokens)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this library runs on a single MI355X)")
         return 2
+    if args.design is not None:
+        return run_design(args)
 
     from xeno_rt_amd.config import parse_config
     from xeno_rt_amd.engine import Engine

@@ -44,15 +44,14 @@ class Attention(Mixer):
                  convolution=None, names: Optional[Dict[str, str]] = None):
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
             raise ValueError(f"head counts {n_heads}/{n_kv_heads}: the first must be a multiple of the second")
-        rotates = position is not None and position.rotation() is not None
-        if head_dim <= 0 or (rotates and head_dim % 2 != 0):          # llama.rs:125-128 takes any size; a rotation pairs dims, so an even one
-            raise ValueError(f"head_dim {head_dim} must be positive and even")
         self.value_dim = head_dim if value_dim is None else int(value_dim)
         self.sink = bool(sink)
         self.convolution = convolution
         self.general = self.sink or self.value_dim != head_dim or convolution is not None
-        if self.general and (qk_norm or rotates):
-            raise ValueError("attention with a sink, a convolution or values of another width takes neither head norms nor a rotation")
+        if head_dim <= 0 or (head_dim % 2 != 0 and not self.general):   # llama.rs:125-128 takes any size; the rotation pairs dims, so an even one
+            raise ValueError(f"head_dim {head_dim} must be positive and even")
+        if self.general and qk_norm:
+            raise ValueError("attention with a sink, a convolution or values of another width takes no head norms")
         self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                       "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", **(names or {})}
         self.prefix = prefix
@@ -99,6 +98,8 @@ class Attention(Mixer):
         if self.position is not None:
             self.position.bind(tensors, runtime)
         if self.general:
+            if self.position is not None and self.position.rotation() is not None:
+                raise ValueError("attention with a sink, a convolution or values of another width takes no rotation")
             if self.convolution is not None:
                 self.convolution.bind(tensors, runtime)
             self.w_qkv = runtime.weight([tensors[p + n[name]] for name in "qkv"])
