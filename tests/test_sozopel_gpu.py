@@ -5,7 +5,9 @@ generation through the library's loop; and every new mechanism alone against pla
 that a window's edge, a far state or a sink shows.
 
 In 32-bit the kernels work a sequence off in its own order whatever the step looks like, so logits are also compared
-bit for bit between schedules."""
+bit for bit between schedules, as long as no step brings a sequence more than 64 tokens: a longer portion is cut into
+segments whose recurrent states are worked out side by side and joined afterwards, the same sums in another order,
+and is compared within the sums' rounding instead."""
 import math
 
 import pytest
@@ -70,6 +72,10 @@ def engines(models):
     return get
 
 
+def same_but_for_rounding(got, want):
+    return float((got - want).abs().max()) <= 2e-5 * float(want.abs().max())
+
+
 def in_portions(engine, ids, sizes):
     """The request alone, cut into steps of the given sizes (the last size repeats); logits of every token."""
     slot = engine.alloc_slot()
@@ -106,7 +112,8 @@ def test_token_by_token_from_the_first(name, dtype, models, engines):
     got = in_portions(engine, ids, [1])
     assert_logits(got, want, dtype, f"sozopel {name} token by token, first bad row {first_bad_position(got, want, dtype)}")
     if dtype == "float32":
-        assert torch.equal(got, run_whole(engine, ids)), "a decoded token differs from the same token in a prompt"
+        assert same_but_for_rounding(got, run_whole(engine, ids)), "a decoded token differs from the same token in a prompt"
+        assert torch.equal(got[:60], run_whole(engine, ids[:60])), "a decoded token's bits differ from the same token's in a short prompt"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -118,7 +125,9 @@ def test_portions(name, sizes, dtype, models, engines):
     got = in_portions(engine, ids, sizes)
     assert_logits(got, want, dtype, f"sozopel {name} portions {sizes}, first bad row {first_bad_position(got, want, dtype)}")
     if dtype == "float32":
-        assert torch.equal(got, run_whole(engine, ids)), f"portions {sizes} change the bits"
+        assert same_but_for_rounding(got, run_whole(engine, ids)), f"portions {sizes} change more than the rounding"
+        if max(sizes) <= 64:
+            assert torch.equal(got, in_portions(engine, ids, [1])), f"portions {sizes} change the bits"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -136,7 +145,9 @@ def test_unequal_batches_through_reused_slots(name, dtype, models, engines):
         for index, (g, w) in enumerate(zip(got, wants)):
             assert_logits(g, w, dtype, f"sozopel {name} batch {prompts} request {index}, first bad row {first_bad_position(g, w, dtype)}")
             if dtype == "float32":
-                assert torch.equal(g, run_whole(engine, requests[index])), "a request's bits depend on its batch"
+                assert same_but_for_rounding(g, run_whole(engine, requests[index])), "a request depends on its batch"
+                if max(prompts) <= 64:
+                    assert torch.equal(g, in_portions(engine, requests[index], [1])), "a request's bits depend on its batch"
     engine.cache.check()
 
 
@@ -294,10 +305,39 @@ def test_linear_recurrence_in_its_three_forms(heads, dim, vdim, dtype, ops):
             limit = 2e-5 if dtype == torch.float32 else 2e-2
             assert float((got - want).abs().max()) <= limit * float(want.abs().max()), f"{what}, cuts {cuts[:4]}"
             assert float(state[0].abs().max()) == 0.0, "another sequence's state was touched"
+            if max(cuts) > 64:                       # (segments side by side: the same sums in another order)
+                continue
             if first is None:
                 first = (got, state.clone())
             else:
                 assert torch.equal(got, first[0]) and torch.equal(state, first[1]), f"{what}: cuts {cuts[:4]} change the bits"
+
+
+def test_recurrence_of_unequal_sequences_in_one_step(ops):
+    """Sequences of 200, 65 and 3 tokens and one that is padding, in one step (the long ones in several segments) and then one
+    more token each: every sequence as it is alone, and the padding's rows zeros."""
+    heads, dim, vdim, lengths = 2, 24, 40, [200, 65, 3]
+    generator = torch.Generator().manual_seed(8)
+    total = sum(lengths) + 2
+    q, k = torch.randn(total + 3, heads * dim, generator=generator), torch.randn(total + 3, heads * dim, generator=generator)
+    v, z = torch.randn(total + 3, heads * vdim, generator=generator), torch.randn(total + 3, heads * dim, generator=generator)
+    options = dict(decay_mode="sigmoid_power", decay_power=0.25, norm_eps=1e-5)
+    state = torch.zeros(5, heads, dim, vdim, device="cuda")
+    out = torch.empty(total, heads * vdim, device="cuda")
+    step = Step([3, -1, 1, 4], [lengths[0], 2, lengths[1], lengths[2]], [0, 0, 0, 0])
+    ops.linear_recurrence(q[:total].cuda(), k[:total].cuda(), v[:total].cuda(), state, step, out, heads, dim, vdim, z[:total].cuda(), **options)
+    more = torch.empty(3, heads * vdim, device="cuda")
+    ops.linear_recurrence(q[total:].cuda(), k[total:].cuda(), v[total:].cuda(), state, Step([3, 1, 4], [1, 1, 1], lengths), more,
+                          heads, dim, vdim, z[total:].cuda(), **options)
+    assert float(out[200:202].abs().max()) == 0.0 and float(state[0].abs().max()) == 0.0 and float(state[2].abs().max()) == 0.0
+    begins = [0, 202, 267]
+    for index, (begin, length) in enumerate(zip(begins, lengths)):
+        rows = list(range(begin, begin + length)) + [total + index]
+        qd, kd, vd = (t[rows].double().reshape(length + 1, heads, -1) for t in (q, k, v))
+        decay = torch.sigmoid(z[rows].double()).pow(0.25).reshape(length + 1, heads, dim)
+        want = P.rms_divide(P.recurrence(qd, kd, vd, decay), 1e-5).reshape(length + 1, -1)
+        got = torch.cat([out[begin:begin + length], more[index:index + 1]]).double().cpu()
+        assert float((got - want).abs().max()) <= 2e-5 * float(want.abs().max()), f"sequence {index}"
 
 
 def test_a_state_keeps_a_token_from_far_back(ops):

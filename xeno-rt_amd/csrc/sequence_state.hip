@@ -106,105 +106,223 @@ __global__ void __launch_bounds__(CONV_THREADS) short_conv_kernel(
 }
 
 // ---- linear recurrence -----------------------------------------------------------------------------------------
+// A wavefront owns 64 columns of one head's state, a lane one column: S[0 .. dim) in registers. The token's q, k and decays
+// lie across the lanes (lane l holds channels l, l + 64, ...), are brought into their final form there (scales, the decay's
+// exponentials), and reach the products as scalar operands, one lane's value at a time; the next token's loads are on their
+// way meanwhile. A long prompt is cut into segments of tokens that run side by side: first every segment but a sequence's
+// last works out what it adds to the state from empty hands (L) and the product of its decays (P); then the states at the
+// segments' beginnings follow from S <- P S + L in their order; then every segment runs again from its true state and
+// writes the outputs. The heads' norm, weight and gate are a pass of their own over the raw outputs.
 
-constexpr int REC_CHUNK = 16;             // tokens whose q, k and decays are staged in LDS at a time (fewer where heads are large)
+constexpr int REC_SEGMENT = 64;           // fewest tokens of a segment
+constexpr int REC_WAVES_WANTED = 2048;    // segments are made until the launch has about this many wavefronts
 
-template <int DIM, bool BONUS, int THREADS>
-__global__ void __launch_bounds__(THREADS) recurrence_kernel(const xrt_recurrence a, int dtype, const int* __restrict__ seq_offsets,
-                                                             const int* __restrict__ seq_slots, int chunk) {
-    extern __shared__ float lds[];
-    constexpr int ARRAYS = BONUS ? 4 : 3;                  // q, k, decay and, with a bonus, bonus * k
-    const int seq = blockIdx.x, head = blockIdx.y, j = threadIdx.x;
-    const int lane = threadIdx.x % XRT_WAVE, wave = threadIdx.x / XRT_WAVE, waves = blockDim.x / XRT_WAVE;
-    const int begin = seq_offsets[seq], end = seq_offsets[seq + 1], slot = seq_slots[seq];
+struct RecurrencePlan {
+    int vslices, segment, segments;       // wavefronts per head; tokens per segment; segments of the longest sequence
+    long raw_floats, state_floats, decay_floats;
+};
+
+RecurrencePlan recurrence_plan(int n_seqs, int max_count, long tokens, int heads, int dim, int vdim) {
+    RecurrencePlan p;
+    p.vslices = (vdim + XRT_WAVE - 1) / XRT_WAVE;
+    const long row = (long)max(1, n_seqs) * heads * p.vslices;
+    const long wanted = max(1L, (REC_WAVES_WANTED + row - 1) / row);
+    const long length = (max_count + wanted - 1) / wanted;
+    p.segment = (int)max((long)REC_SEGMENT, (length + 15) / 16 * 16);
+    p.segments = max(1, (max_count + p.segment - 1) / p.segment);
+    p.raw_floats = tokens * heads * vdim;
+    p.state_floats = p.segments > 1 ? (long)n_seqs * (p.segments + 1) * heads * dim * vdim : 0;
+    p.decay_floats = p.segments > 1 ? (long)n_seqs * p.segments * heads * dim : 0;
+    return p;
+}
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// What a token brings, across the lanes: channel lane + 64 m in element m. Channels beyond dim read as q = k = 0, decay = 1.
+template <int M>
+struct TokenInputs {
+    float q[M], k[M], d[M], v, bonus_dot;
+};
+
+template <int M, bool BONUS>
+__device__ __forceinline__ void load_token(TokenInputs<M>& in, const xrt_recurrence& a, int dtype, long row, int head, int column, bool owner) {
+    const int lane = threadIdx.x;
+    float dot = 0.f;
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+        const int i = lane + XRT_WAVE * m;
+        in.q[m] = 0.f; in.k[m] = 0.f; in.d[m] = 1.f;
+        if (i < a.dim) {
+            const long at = (long)head * a.dim + i;
+            in.q[m] = load_as_float(a.q, dtype, row * a.q_stride + at) * a.q_scale;
+            in.k[m] = load_as_float(a.k, dtype, row * a.k_stride + at) * a.k_scale;
+            if (a.decay_mode == XRT_DECAY_PER_HEAD) {
+                in.d[m] = a.decay[head];
+            } else {
+                float z = a.decay[row * (long)a.heads * a.dim + at];
+                if (a.decay_bias != nullptr) z += load_as_float(a.decay_bias, a.decay_bias_dtype, at);
+                if (a.decay_mode == XRT_DECAY_EXP_NEG_EXP) in.d[m] = expf(-expf(z));
+                else if (a.decay_mode == XRT_DECAY_SIGMOID_POWER) in.d[m] = expf(-softplus_exact(-z) * a.decay_power);   // sigmoid(z)^power
+                else in.d[m] = z;
+            }
+            if constexpr (BONUS) dot = fmaf(load_as_float(a.bonus, a.bonus_dtype, at) * in.k[m], in.q[m], dot);
+        }
+    }
+    in.v = owner ? load_as_float(a.v, dtype, row * a.v_stride + (long)head * a.vdim + column) : 0.f;
+    in.bonus_dot = BONUS ? wave_sum(dot) : 0.f;            // sum over the channels of bonus * k * q: what the token's own k v^T adds to its output
+}
+
+// grid (sequences, heads * vslices, segments), one wavefront each.
+// FINAL false: a segment from empty hands, no outputs: its L to states[seq][segment], its P to decays[seq][segment].
+// FINAL true: from the state at the segment's beginning (the cache's for a sequence in one segment, else states[...]: entry
+// `segments` for the first segment, entry c - 1 for segment c), raw outputs to raw [tokens][heads * vdim]; a sequence's last
+// segment leaves the state in the cache.
+template <int DIM, bool BONUS, bool FINAL>
+__global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurrence a, int dtype, const int* __restrict__ seq_offsets,
+                                                             const int* __restrict__ seq_slots, int segment, int segments, int vslices,
+                                                             float* __restrict__ states, float* __restrict__ decays, float* __restrict__ raw) {
+    constexpr int M = (DIM + XRT_WAVE - 1) / XRT_WAVE;
+    const int seq = blockIdx.x, head = blockIdx.y / vslices, vslice = blockIdx.y % vslices, lane = threadIdx.x;
+    const int begin = seq_offsets[seq], count = seq_offsets[seq + 1] - begin, slot = seq_slots[seq];
+    const int first = blockIdx.z * segment, last = min(count, first + segment);
+    if (first >= count) return;
     const int dim = a.dim, vdim = a.vdim, heads = a.heads;
-    const long out_width = (long)heads * vdim;
+    const int column = vslice * XRT_WAVE + lane;
+    const bool owner = column < vdim;
+    const bool ends_sequence = last == count, whole = count <= segment;
+    if (!FINAL && ends_sequence) return;                   // nobody asks what a sequence's last segment adds
     if (slot < 0) {
-        for (int t = begin; t < end; ++t)
-            for (int c = j; c < vdim; c += blockDim.x) store_from_float(a.out, dtype, t * out_width + (long)head * vdim + c, 0.f);
+        if (FINAL && owner)
+            for (int t = first; t < last; ++t) raw[(long)(begin + t) * heads * vdim + (long)head * vdim + column] = 0.f;
         return;
     }
-    float* staged = lds;                                   // [chunk][ARRAYS][dim]
-    float* raw = lds + chunk * ARRAYS * dim;               // [chunk][vdim]
-    const bool owner = j < vdim;
-    float* kept = a.state + (((long)slot * heads + head) * dim) * vdim + j;
+    const long per_head = (long)dim * vdim;
+    float* cached = a.state + ((long)slot * heads + head) * per_head + column;
+    float* at_segment = states + (((long)seq * (segments + 1) + blockIdx.z) * heads + head) * per_head + column;
     float S[DIM];
+    if (FINAL) {
+        const float* from = whole ? cached
+                                  : states + (((long)seq * (segments + 1) + (blockIdx.z == 0 ? segments : blockIdx.z - 1)) * heads + head) * per_head + column;
 #pragma unroll
-    for (int i = 0; i < DIM; ++i) S[i] = owner && i < dim ? kept[(long)i * vdim] : 0.f;
-    for (int t0 = begin; t0 < end; t0 += chunk) {
-        const int n = min(chunk, end - t0);
-        __syncthreads();                                   // the chunk before is read to its end
-        for (int e = threadIdx.x; e < n * dim; e += blockDim.x) {
-            const int tt = e / dim, i = e % dim;
-            const long row = t0 + tt, at = (long)head * dim + i;
-            const float qv = load_as_float(a.q, dtype, row * a.q_stride + at) * a.q_scale;
-            const float kv = load_as_float(a.k, dtype, row * a.k_stride + at) * a.k_scale;
-            float decay;
-            if (a.decay_mode == XRT_DECAY_PER_HEAD) {
-                decay = a.decay[head];
-            } else {
-                float z = a.decay[row * (long)heads * dim + at];
-                if (a.decay_bias != nullptr) z += load_as_float(a.decay_bias, a.decay_bias_dtype, at);
-                if (a.decay_mode == XRT_DECAY_EXP_NEG_EXP) decay = expf(-expf(z));
-                else if (a.decay_mode == XRT_DECAY_SIGMOID_POWER) decay = expf(-softplus_exact(-z) * a.decay_power);   // sigmoid(z)^power
-                else decay = z;
-            }
-            float* to = staged + (long)tt * ARRAYS * dim + i;
-            to[0] = qv;
-            to[dim] = kv;
-            to[2 * dim] = decay;
-            if constexpr (BONUS) to[3 * dim] = load_as_float(a.bonus, a.bonus_dtype, at) * kv;
-        }
-        float v_now = owner ? load_as_float(a.v, dtype, (long)t0 * a.v_stride + (long)head * vdim + j) : 0.f;
-        __syncthreads();
-        for (int tt = 0; tt < n; ++tt) {
-            const float v_next = owner && tt + 1 < n ? load_as_float(a.v, dtype, (long)(t0 + tt + 1) * a.v_stride + (long)head * vdim + j) : 0.f;
-            const float* sq = staged + (long)tt * ARRAYS * dim;
-            const float* sk = sq + dim;
-            const float* sd = sq + 2 * dim;
-            float o[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < DIM; ++i) S[i] = owner && i < dim ? from[(long)i * vdim] : 0.f;
+    } else {
 #pragma unroll
-            for (int i = 0; i < DIM; ++i) {
-                if (i < dim) {
-                    const float kv = sk[i] * v_now;
-                    if constexpr (BONUS) {
-                        o[i % 4] = fmaf(fmaf(sq[3 * dim + i], v_now, S[i]), sq[i], o[i % 4]);
-                        S[i] = fmaf(sd[i], S[i], kv);
+        for (int i = 0; i < DIM; ++i) S[i] = 0.f;
+    }
+    float product[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) product[m] = 1.f;
+
+    TokenInputs<M> now, next;
+    load_token<M, BONUS>(now, a, dtype, begin + first, head, column, owner);
+    for (int t = first; t < last; ++t) {
+        if (t + 1 < last) load_token<M, BONUS>(next, a, dtype, begin + t + 1, head, column, owner);
+        float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int g = 0; g < DIM / 16; ++g) {
+            if (g * 16 < dim) {                            // (channels from dim up to the next multiple of 16 hold zeros and stay zero)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int i = g * 16 + e;
+                    const float s_k = lane_value(now.k[i / XRT_WAVE], i % XRT_WAVE);
+                    const float s_d = lane_value(now.d[i / XRT_WAVE], i % XRT_WAVE);
+                    const float kv = s_k * now.v;
+                    if constexpr (FINAL) {
+                        const float s_q = lane_value(now.q[i / XRT_WAVE], i % XRT_WAVE);
+                        if constexpr (BONUS) {             // the token reads the state as the tokens before it left it
+                            o[e % 4] = fmaf(S[i], s_q, o[e % 4]);
+                            S[i] = fmaf(s_d, S[i], kv);
+                        } else {
+                            S[i] = fmaf(s_d, S[i], kv);
+                            o[e % 4] = fmaf(S[i], s_q, o[e % 4]);
+                        }
                     } else {
-                        S[i] = fmaf(sd[i], S[i], kv);
-                        o[i % 4] = fmaf(S[i], sq[i], o[i % 4]);
+                        S[i] = fmaf(s_d, S[i], kv);
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);         // (one group's scalars at a time: all of a token's would not fit the scalar registers)
             }
-            if (owner) raw[tt * vdim + j] = (o[0] + o[1]) + (o[2] + o[3]);
-            v_now = v_next;
         }
-        __syncthreads();
-        // the heads' outputs of the chunk: norm over vdim, weight, gate; a wavefront a token
-        for (int tt = wave; tt < n; tt += waves) {
-            const long row = t0 + tt;
-            float inv = 1.f;
-            if (a.norm) {
-                float squares = 0.f;
-                for (int c = lane; c < vdim; c += XRT_WAVE) squares = fmaf(raw[tt * vdim + c], raw[tt * vdim + c], squares);
-                inv = 1.0f / sqrtf(wave_sum(squares) / (float)vdim + a.eps);
-            }
-            for (int c = lane; c < vdim; c += XRT_WAVE) {
-                float value = raw[tt * vdim + c] * inv;
-                if (a.norm_weight != nullptr)
-                    value *= load_as_float(a.norm_weight, a.norm_weight_dtype, a.norm_weight_per_head ? (long)head * vdim + c : c);
-                if (a.gate != nullptr) {
-                    const float g = load_as_float(a.gate, dtype, row * a.gate_stride + (long)head * vdim + c);
-                    value *= a.gate_act == XRT_GATE_SILU ? silu_exact(g) : g;
-                }
-                store_from_float(a.out, dtype, row * out_width + (long)head * vdim + c, value);
-            }
+        if constexpr (FINAL) {
+            float out = (o[0] + o[1]) + (o[2] + o[3]);
+            if constexpr (BONUS) out = fmaf(now.bonus_dot, now.v, out);
+            if (owner) raw[(long)(begin + t) * heads * vdim + (long)head * vdim + column] = out;
+        } else {
+#pragma unroll
+            for (int m = 0; m < M; ++m) product[m] *= now.d[m];
+        }
+        now = next;
+    }
+    if (FINAL) {
+        if (ends_sequence && owner) {
+#pragma unroll
+            for (int i = 0; i < DIM; ++i)
+                if (i < dim) cached[(long)i * vdim] = S[i];
+        }
+    } else {
+        if (owner) {
+#pragma unroll
+            for (int i = 0; i < DIM; ++i)
+                if (i < dim) at_segment[(long)i * vdim] = S[i];
+        }
+        if (vslice == 0) {
+#pragma unroll
+            for (int m = 0; m < M; ++m)
+                if (lane + XRT_WAVE * m < dim)
+                    decays[(((long)seq * segments + blockIdx.z) * heads + head) * dim + lane + XRT_WAVE * m] = product[m];
         }
     }
-    if (owner) {
-#pragma unroll
-        for (int i = 0; i < DIM; ++i)
-            if (i < dim) kept[(long)i * vdim] = S[i];
+}
+
+// The states at the segments' beginnings, in place of what the segments add: entry `segments` takes the cache's state (the first
+// segment's), entry c what segment c + 1 starts from. grid (sequences, heads * vslices), a lane a column.
+__global__ void __launch_bounds__(XRT_WAVE) recurrence_combine_kernel(const xrt_recurrence a, const int* __restrict__ seq_offsets,
+                                                                     const int* __restrict__ seq_slots, int segment, int segments, int vslices,
+                                                                     float* __restrict__ states, const float* __restrict__ decays) {
+    const int seq = blockIdx.x, head = blockIdx.y / vslices, column = blockIdx.y % vslices * XRT_WAVE + threadIdx.x;
+    const int count = seq_offsets[seq + 1] - seq_offsets[seq], slot = seq_slots[seq];
+    if (slot < 0 || count <= segment || column >= a.vdim) return;
+    const int mine = (count + segment - 1) / segment;      // this sequence's segments
+    const long per_head = (long)a.dim * a.vdim;
+    const float* cached = a.state + ((long)slot * a.heads + head) * per_head + column;
+    for (int i = 0; i < a.dim; ++i) {
+        float s = cached[(long)i * a.vdim];
+        states[(((long)seq * (segments + 1) + segments) * a.heads + head) * per_head + (long)i * a.vdim + column] = s;
+        for (int c = 0; c + 1 < mine; ++c) {
+            float* entry = states + (((long)seq * (segments + 1) + c) * a.heads + head) * per_head + (long)i * a.vdim + column;
+            s = fmaf(decays[(((long)seq * segments + c) * a.heads + head) * a.dim + i], s, *entry);
+            *entry = s;
+        }
+    }
+}
+
+// The heads' raw outputs of one token: norm over vdim, weight, gate. A wavefront per (token, head).
+__global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_recurrence a, int dtype, const float* __restrict__ raw,
+                                                                    const int* __restrict__ token_slots) {
+    const long row = blockIdx.x;
+    const int head = blockIdx.y, lane = threadIdx.x, vdim = a.vdim;
+    const long out_at = row * a.heads * vdim + (long)head * vdim;
+    if (token_slots[row] < 0) {
+        for (int c = lane; c < vdim; c += XRT_WAVE) store_from_float(a.out, dtype, out_at + c, 0.f);
+        return;
+    }
+    float inv = 1.f;
+    if (a.norm) {
+        float squares = 0.f;
+        for (int c = lane; c < vdim; c += XRT_WAVE) squares = fmaf(raw[out_at + c], raw[out_at + c], squares);
+        inv = 1.0f / sqrtf(wave_sum(squares) / (float)vdim + a.eps);
+    }
+    for (int c = lane; c < vdim; c += XRT_WAVE) {
+        float value = raw[out_at + c] * inv;
+        if (a.norm_weight != nullptr)
+            value *= load_as_float(a.norm_weight, a.norm_weight_dtype, a.norm_weight_per_head ? (long)head * vdim + c : c);
+        if (a.gate != nullptr) {
+            const float g = load_as_float(a.gate, dtype, row * a.gate_stride + (long)head * vdim + c);
+            value *= a.gate_act == XRT_GATE_SILU ? silu_exact(g) : g;
+        }
+        store_from_float(a.out, dtype, out_at + c, value);
     }
 }
 
@@ -310,41 +428,53 @@ extern "C" int xrt_short_conv(const void* x, int dtype, long tokens, long x_stri
     return 0;
 }
 
+extern "C" long xrt_linear_recurrence_workspace(int n_seqs, int max_count, long tokens, int heads, int dim, int vdim) {
+    if (n_seqs <= 0 || max_count <= 0 || tokens <= 0 || heads <= 0 || dim <= 0 || vdim <= 0) return 0;
+    const RecurrencePlan p = recurrence_plan(n_seqs, max_count, tokens, heads, dim, vdim);
+    return p.raw_floats + p.state_floats + p.decay_floats;
+}
+
 extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, const int* seq_offsets, const int* seq_slots, int n_seqs,
+                                     int max_count, const int* token_slots, long tokens, float* workspace, long workspace_floats,
                                      void* stream) {
-    XRT_REQUIRE(args != nullptr && seq_offsets && seq_slots, "linear_recurrence: null operand");
+    XRT_REQUIRE(args != nullptr && seq_offsets && seq_slots && token_slots, "linear_recurrence: null operand");
     const xrt_recurrence a = *args;
     XRT_REQUIRE(dtype == XRT_F32 || dtype == XRT_BF16, "linear_recurrence: unknown dtype %d", dtype);
     XRT_REQUIRE(a.q && a.k && a.v && a.state && a.out, "linear_recurrence: null operand");
-    XRT_REQUIRE(a.heads > 0 && a.heads <= 65535 && a.dim > 0 && a.dim <= 256 && a.vdim > 0 && a.vdim <= 1024,
-                "linear_recurrence: %d heads of %d x %d: key sizes up to 256 and value sizes up to 1024 are served", a.heads, a.dim, a.vdim);
+    XRT_REQUIRE(a.heads > 0 && a.dim > 0 && a.dim <= 256 && a.vdim > 0 && (long)a.heads * ((a.vdim + XRT_WAVE - 1) / XRT_WAVE) <= 65535,
+                "linear_recurrence: %d heads of %d x %d: key sizes up to 256 are served", a.heads, a.dim, a.vdim);
     XRT_REQUIRE(a.decay_mode >= XRT_DECAY_PER_HEAD && a.decay_mode <= XRT_DECAY_SIGMOID_POWER && a.decay != nullptr,
                 "linear_recurrence: unknown decay mode %d, or no decays", a.decay_mode);
     XRT_REQUIRE(a.q_stride >= a.heads * a.dim && a.k_stride >= a.heads * a.dim && a.v_stride >= a.heads * a.vdim &&
                 (a.gate == nullptr || a.gate_stride >= a.heads * a.vdim), "linear_recurrence: a row stride is shorter than its heads");
-    if (n_seqs == 0) return 0;
+    XRT_REQUIRE(n_seqs >= 0 && max_count >= 0 && tokens >= 0 && tokens < (1L << 31), "linear_recurrence: bad sizes");
+    if (n_seqs == 0 || tokens == 0 || max_count == 0) return 0;
+    const RecurrencePlan p = recurrence_plan(n_seqs, max_count, tokens, a.heads, a.dim, a.vdim);
+    XRT_REQUIRE(p.segments <= 65535, "linear_recurrence: a step this long is not served");
+    XRT_REQUIRE(workspace != nullptr && workspace_floats >= p.raw_floats + p.state_floats + p.decay_floats,
+                "linear_recurrence: the workspace needs %ld floats", p.raw_floats + p.state_floats + p.decay_floats);
     hipStream_t s = (hipStream_t)stream;
+    float* raw = workspace;
+    float* states = raw + p.raw_floats;
+    float* decays = states + p.state_floats;
     const bool bonus = a.bonus != nullptr;
-    const int threads = (a.vdim + XRT_WAVE - 1) / XRT_WAVE * XRT_WAVE;
-    const size_t per_token = (size_t)((bonus ? 4 : 3) * a.dim + a.vdim) * sizeof(float);
-    const int chunk = (int)min((size_t)REC_CHUNK, (size_t)(64 * 1024) / per_token);           // (at least 5 with the largest heads)
-    const size_t lds = chunk * per_token;
-#define XRT_REC(DIM_, BONUS_, THREADS_) recurrence_kernel<DIM_, BONUS_, THREADS_><<<dim3(n_seqs, a.heads), threads, lds, s>>>(a, dtype, seq_offsets, seq_slots, chunk)
-    // (a workgroup of few wavefronts may keep a whole column of a large state in registers)
-#define XRT_REC_THREADS(DIM_, BONUS_)                                                            \
-    do {                                                                                         \
-        if (threads <= 128) XRT_REC(DIM_, BONUS_, 128); else if (threads <= 256) XRT_REC(DIM_, BONUS_, 256); \
-        else XRT_REC(DIM_, BONUS_, 1024);                                                        \
+    const dim3 grid(n_seqs, a.heads * p.vslices, p.segments);
+#define XRT_REC(DIM_, BONUS_, FINAL_) recurrence_kernel<DIM_, BONUS_, FINAL_><<<grid, XRT_WAVE, 0, s>>>(a, dtype, seq_offsets, seq_slots, \
+        p.segment, p.segments, p.vslices, states, decays, raw)
+#define XRT_REC_DIM(BONUS_, FINAL_)                                                                \
+    do {                                                                                           \
+        if (a.dim <= 32) XRT_REC(32, BONUS_, FINAL_); else if (a.dim <= 64) XRT_REC(64, BONUS_, FINAL_); \
+        else if (a.dim <= 128) XRT_REC(128, BONUS_, FINAL_); else XRT_REC(256, BONUS_, FINAL_);    \
     } while (0)
-#define XRT_REC_DIM(BONUS_)                                                                      \
-    do {                                                                                         \
-        if (a.dim <= 32) XRT_REC_THREADS(32, BONUS_); else if (a.dim <= 64) XRT_REC_THREADS(64, BONUS_); \
-        else if (a.dim <= 128) XRT_REC_THREADS(128, BONUS_); else XRT_REC_THREADS(256, BONUS_);  \
-    } while (0)
-    if (bonus) XRT_REC_DIM(true); else XRT_REC_DIM(false);
+    if (p.segments > 1) {
+        XRT_REC_DIM(false, false);                         // (what a segment adds to the state does not know of the bonus)
+        recurrence_combine_kernel<<<dim3(n_seqs, a.heads * p.vslices), XRT_WAVE, 0, s>>>(a, seq_offsets, seq_slots, p.segment, p.segments,
+                                                                                        p.vslices, states, decays);
+    }
+    if (bonus) XRT_REC_DIM(true, true); else XRT_REC_DIM(false, true);
 #undef XRT_REC_DIM
-#undef XRT_REC_THREADS
 #undef XRT_REC
+    recurrence_finish_kernel<<<dim3((unsigned)tokens, a.heads), XRT_WAVE, 0, s>>>(a, dtype, raw, token_slots);
     XRT_LAUNCH_CHECK("linear_recurrence");
     return 0;
 }

@@ -225,7 +225,11 @@ typedef struct {
     int gate_act;
     void* out;
 } xrt_recurrence;
-int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, const int* seq_offsets, const int* seq_slots, int n_seqs, void* stream);
+// token_slots [tokens]: the slot of every token's sequence. The workspace holds the raw outputs and, where a long prompt is cut
+// into segments that run side by side, the segments' states; xrt_linear_recurrence_workspace says how many floats.
+long xrt_linear_recurrence_workspace(int n_seqs, int max_count, long tokens, int heads, int dim, int vdim);
+int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, const int* seq_offsets, const int* seq_slots, int n_seqs,
+                          int max_count, const int* token_slots, long tokens, float* workspace, long workspace_floats, void* stream);
 
 // residual[r] += scale * (x0[r] / rms(x0[r]) * gain0 + x1[r] / rms(x1[r]) * gain1); x float32 [rows][width], x1 may be null
 int xrt_add_normed(float* residual, const float* x0, const void* gain0, const float* x1, const void* gain1, int gain_dtype,

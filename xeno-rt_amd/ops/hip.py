@@ -192,6 +192,7 @@ class HipOps:
         self.lib.xrt_attention_workspace.restype = ctypes.c_long
         self.lib.xrt_probe_read_bytes.restype = ctypes.c_long
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
+        self.lib.xrt_linear_recurrence_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
     def _check(self, status: int) -> None:
@@ -607,7 +608,12 @@ class HipOps:
         self._require(out, "recurrence out", q.dtype, (tokens, heads * vdim), q)
         record.out = out.data_ptr()
         offsets, slots, n = self._sequences(batch, tokens, q)
-        self._check(self.lib.xrt_linear_recurrence(ctypes.byref(record), _code(q), offsets, slots, n, self._stream(q)))
+        self._require(batch.slots, "slots", torch.int32, (tokens,), q)
+        need = int(self.lib.xrt_linear_recurrence_workspace(n, int(batch.max_count), ctypes.c_long(tokens), heads, dim, vdim))
+        workspace = self._empty(need, torch.float32, q.device)
+        self._check(self.lib.xrt_linear_recurrence(ctypes.byref(record), _code(q), offsets, slots, n, int(batch.max_count),
+                                                   _ptr(batch.slots), ctypes.c_long(tokens), _ptr(workspace), ctypes.c_long(need),
+                                                   self._stream(q)))
 
     def add_normed(self, residual, parts, eps, scale=1.0):
         """residual += scale * sum over (x, gain) in parts of x / sqrt(mean(x^2) + eps) * gain; x float32 like residual; one or two parts."""
