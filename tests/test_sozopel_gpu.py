@@ -5,7 +5,7 @@ generation through the library's loop; and every new mechanism alone against pla
 that a window's edge, a far state or a sink shows.
 
 In 32-bit the kernels work a sequence off in its own order whatever the step looks like, so logits are also compared
-bit for bit between schedules, as long as no step brings a sequence more than 64 tokens: a longer portion is cut into
+bit for bit between schedules, as long as no step brings a sequence more than 32 tokens: a longer portion is cut into
 segments whose recurrent states are worked out side by side and joined afterwards, the same sums in another order,
 and is compared within the sums' rounding instead."""
 import math
@@ -113,7 +113,7 @@ def test_token_by_token_from_the_first(name, dtype, models, engines):
     assert_logits(got, want, dtype, f"sozopel {name} token by token, first bad row {first_bad_position(got, want, dtype)}")
     if dtype == "float32":
         assert same_but_for_rounding(got, run_whole(engine, ids)), "a decoded token differs from the same token in a prompt"
-        assert torch.equal(got[:60], run_whole(engine, ids[:60])), "a decoded token's bits differ from the same token's in a short prompt"
+        assert torch.equal(got[:30], run_whole(engine, ids[:30])), "a decoded token's bits differ from the same token's in a short prompt"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -126,7 +126,7 @@ def test_portions(name, sizes, dtype, models, engines):
     assert_logits(got, want, dtype, f"sozopel {name} portions {sizes}, first bad row {first_bad_position(got, want, dtype)}")
     if dtype == "float32":
         assert same_but_for_rounding(got, run_whole(engine, ids)), f"portions {sizes} change more than the rounding"
-        if max(sizes) <= 64:
+        if max(sizes) <= 32:
             assert torch.equal(got, in_portions(engine, ids, [1])), f"portions {sizes} change the bits"
 
 
@@ -146,7 +146,7 @@ def test_unequal_batches_through_reused_slots(name, dtype, models, engines):
             assert_logits(g, w, dtype, f"sozopel {name} batch {prompts} request {index}, first bad row {first_bad_position(g, w, dtype)}")
             if dtype == "float32":
                 assert same_but_for_rounding(g, run_whole(engine, requests[index])), "a request depends on its batch"
-                if max(prompts) <= 64:
+                if max(prompts) <= 32:
                     assert torch.equal(g, in_portions(engine, requests[index], [1])), "a request's bits depend on its batch"
     engine.cache.check()
 
@@ -305,7 +305,7 @@ def test_linear_recurrence_in_its_three_forms(heads, dim, vdim, dtype, ops):
             limit = 2e-5 if dtype == torch.float32 else 2e-2
             assert float((got - want).abs().max()) <= limit * float(want.abs().max()), f"{what}, cuts {cuts[:4]}"
             assert float(state[0].abs().max()) == 0.0, "another sequence's state was touched"
-            if max(cuts) > 64:                       # (segments side by side: the same sums in another order)
+            if max(cuts) > 32:                       # (segments side by side: the same sums in another order)
                 continue
             if first is None:
                 first = (got, state.clone())

@@ -59,6 +59,10 @@ struct Seen {
 // wavefronts of a workgroup take them side by side (few tokens: a decode step, where one wavefront per (token, head)
 // would leave most of the chip idle): the same sums in the same order, to the bit.
 constexpr int CHUNK_BLOCKS = 8;
+// With a window of up to WINDOW_FOR_SHORT_CHUNKS keys a query sees only a few blocks, and chunks of eight would leave a
+// decode step's eight wavefronts with one or two of them: such a window takes chunks of one block. The choice rests on the
+// window alone, which a model fixes, so every step of a model cuts its keys at the same places.
+constexpr int WINDOW_FOR_SHORT_CHUNKS = 2048;
 
 // `from` merged into `into` (both relative to their own maximum). The products are rounded before they are added
 // (explicit fmaf: what the compiler may contract elsewhere it must not contract differently in two kernels).
@@ -188,7 +192,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads, int head_dim, int value_dim,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
-    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink) {
+    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink, int chunk_blocks) {
     __shared__ float qs[G * OWNED * XRT_WAVE];                 // [G][head_dim]
     __shared__ float ps[WAVES][G * XRT_WAVE];
     // what the wavefronts found in the chunks of a round, for the merge: two sets, used in turn (WAVES > 1)
@@ -217,7 +221,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
     if constexpr (WAVES > 1) __syncthreads(); else wave_sync();
     const int* table = block_table + (long)slot * table_stride;
     const int first_block = first / XRT_BLOCK_TOKENS, last_block = pos / XRT_BLOCK_TOKENS;
-    const int first_chunk = first_block / CHUNK_BLOCKS, last_chunk = last_block / CHUNK_BLOCKS;
+    const int first_chunk = first_block / chunk_blocks, last_chunk = last_block / chunk_blocks;
 
     Seen<OWNED> all[G];
 #pragma unroll
@@ -227,7 +231,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
             Seen<OWNED> here[G];
 #pragma unroll
             for (int g = 0; g < G; ++g) here[g].clear();
-            attend_blocks<T, G, OWNED>(here, max(first_block, chunk * CHUNK_BLOCKS), min(last_block, chunk * CHUNK_BLOCKS + CHUNK_BLOCKS - 1),
+            attend_blocks<T, G, OWNED>(here, max(first_block, chunk * chunk_blocks), min(last_block, chunk * chunk_blocks + chunk_blocks - 1),
                                        first, pos, qs, ps[0], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, value_dim, scale,
                                        biased, slopes, whole_pieces);
 #pragma unroll
@@ -244,7 +248,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
                 Seen<OWNED> here[G];
 #pragma unroll
                 for (int g = 0; g < G; ++g) here[g].clear();
-                attend_blocks<T, G, OWNED>(here, max(first_block, chunk * CHUNK_BLOCKS), min(last_block, chunk * CHUNK_BLOCKS + CHUNK_BLOCKS - 1),
+                attend_blocks<T, G, OWNED>(here, max(first_block, chunk * chunk_blocks), min(last_block, chunk * chunk_blocks + chunk_blocks - 1),
                                            first, pos, qs, ps[wave], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, value_dim, scale,
                                            biased, slopes, whole_pieces);
 #pragma unroll
@@ -307,11 +311,12 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
     const int row_width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim;
     // few (token, head) pairs (a decode step): a workgroup of wavefronts each, which take the chunks of keys side by side
     const bool side_by_side = (long)tokens * n_heads <= 8L * XRT_COMPUTE_UNITS;
+    const int chunk_blocks = window > 0 && window <= WINDOW_FOR_SHORT_CHUNKS ? 1 : CHUNK_BLOCKS;
     const size_t round_bytes = (size_t)2 * CHUNK_WAVES * together * value_dim * sizeof(float);
 #define XRT_GENERIC(T, WAVES_, G_, OWNED_)                                                                                \
     attention_generic_kernel<T, WAVES_, G_, OWNED_><<<(unsigned)items, WAVES_ * XRT_WAVE, WAVES_ > 1 ? round_bytes : 0, s>>>( \
         (const T*)qkv, row_width, n_heads, n_kv_heads, head_dim, value_dim, (const T*)k_cache, (const T*)v_cache, block_table,       \
-        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink)
+        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink, chunk_blocks)
 #define XRT_GENERIC_WAVES(T, G_, OWNED_) do { if (side_by_side) XRT_GENERIC(T, CHUNK_WAVES, G_, OWNED_); else XRT_GENERIC(T, 1, G_, OWNED_); } while (0)
 #define XRT_GENERIC_SETS(T)                                                                                               \
     do {                                                                                                                  \

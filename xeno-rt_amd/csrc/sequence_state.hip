@@ -30,7 +30,7 @@ __device__ __forceinline__ float softplus_exact(float z) { return fmaxf(z, 0.f) 
 // ---- short convolution -----------------------------------------------------------------------------------------
 
 constexpr int CONV_MAX_TAPS = 8;
-constexpr int CONV_SEGMENT = 64;          // tokens of a sequence that one workgroup walks
+constexpr int CONV_SEGMENT = 16;          // tokens of a sequence that one workgroup walks
 constexpr int CONV_THREADS = 256;         // channels of a workgroup
 
 // Input `at` (counted from the step's first token of the sequence; negative: before the step) of channel c.
@@ -114,8 +114,8 @@ __global__ void __launch_bounds__(CONV_THREADS) short_conv_kernel(
 // segments' beginnings follow from S <- P S + L in their order; then every segment runs again from its true state and
 // writes the outputs. The heads' norm, weight and gate are a pass of their own over the raw outputs.
 
-constexpr int REC_SEGMENT = 64;           // fewest tokens of a segment
-constexpr int REC_WAVES_WANTED = 2048;    // segments are made until the launch has about this many wavefronts
+constexpr int REC_SEGMENT = 32;           // fewest tokens of a segment
+constexpr int REC_WAVES_WANTED = 4096;    // segments are made until the launch has about this many wavefronts (a few to every SIMD)
 
 struct RecurrencePlan {
     int vslices, segment, segments;       // wavefronts per head; tokens per segment; segments of the longest sequence
@@ -223,6 +223,8 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurren
 #pragma unroll
         for (int g = 0; g < DIM / 16; ++g) {
             if (g * 16 < dim) {                            // (channels from dim up to the next multiple of 16 hold zeros and stay zero)
+                // (the group's scalars are taken from the lanes here and not earlier: all of a token's would not fit the scalar registers)
+                asm volatile("" : "+v"(now.q[g * 16 / XRT_WAVE]), "+v"(now.k[g * 16 / XRT_WAVE]), "+v"(now.d[g * 16 / XRT_WAVE]));
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int i = g * 16 + e;
@@ -277,23 +279,34 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurren
 }
 
 // The states at the segments' beginnings, in place of what the segments add: entry `segments` takes the cache's state (the first
-// segment's), entry c what segment c + 1 starts from. grid (sequences, heads * vslices), a lane a column.
+// segment's), entry c what segment c + 1 starts from. grid (sequences, heads * vslices, dim): a wavefront a row of the state,
+// a lane a column; the segments' additions are fetched eight at a time before the chain of products that needs them.
 __global__ void __launch_bounds__(XRT_WAVE) recurrence_combine_kernel(const xrt_recurrence a, const int* __restrict__ seq_offsets,
                                                                      const int* __restrict__ seq_slots, int segment, int segments, int vslices,
                                                                      float* __restrict__ states, const float* __restrict__ decays) {
-    const int seq = blockIdx.x, head = blockIdx.y / vslices, column = blockIdx.y % vslices * XRT_WAVE + threadIdx.x;
+    const int seq = blockIdx.x, head = blockIdx.y / vslices, column = blockIdx.y % vslices * XRT_WAVE + threadIdx.x, i = blockIdx.z;
     const int count = seq_offsets[seq + 1] - seq_offsets[seq], slot = seq_slots[seq];
     if (slot < 0 || count <= segment || column >= a.vdim) return;
     const int mine = (count + segment - 1) / segment;      // this sequence's segments
-    const long per_head = (long)a.dim * a.vdim;
-    const float* cached = a.state + ((long)slot * a.heads + head) * per_head + column;
-    for (int i = 0; i < a.dim; ++i) {
-        float s = cached[(long)i * a.vdim];
-        states[(((long)seq * (segments + 1) + segments) * a.heads + head) * per_head + (long)i * a.vdim + column] = s;
-        for (int c = 0; c + 1 < mine; ++c) {
-            float* entry = states + (((long)seq * (segments + 1) + c) * a.heads + head) * per_head + (long)i * a.vdim + column;
-            s = fmaf(decays[(((long)seq * segments + c) * a.heads + head) * a.dim + i], s, *entry);
-            *entry = s;
+    const long per_head = (long)a.dim * a.vdim, within = (long)i * a.vdim + column;
+    float s = a.state[((long)slot * a.heads + head) * per_head + within];
+    float* entries = states + ((long)seq * (segments + 1) * a.heads + head) * per_head + within;      // entry c: + c * heads * per_head
+    const float* products = decays + ((long)seq * segments * a.heads + head) * a.dim + i;               // of segment c: + c * heads * dim
+    entries[(long)segments * a.heads * per_head] = s;
+    for (int c0 = 0; c0 + 1 < mine; c0 += 8) {
+        float added[8], decay[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const bool there = c0 + e + 1 < mine;
+            added[e] = there ? entries[(long)(c0 + e) * a.heads * per_head] : 0.f;
+            decay[e] = there ? products[(long)(c0 + e) * a.heads * a.dim] : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            if (c0 + e + 1 < mine) {
+                s = fmaf(decay[e], s, added[e]);
+                entries[(long)(c0 + e) * a.heads * per_head] = s;
+            }
         }
     }
 }
@@ -468,7 +481,7 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
     } while (0)
     if (p.segments > 1) {
         XRT_REC_DIM(false, false);                         // (what a segment adds to the state does not know of the bonus)
-        recurrence_combine_kernel<<<dim3(n_seqs, a.heads * p.vslices), XRT_WAVE, 0, s>>>(a, seq_offsets, seq_slots, p.segment, p.segments,
+        recurrence_combine_kernel<<<dim3(n_seqs, a.heads * p.vslices, a.dim), XRT_WAVE, 0, s>>>(a, seq_offsets, seq_slots, p.segment, p.segments,
                                                                                         p.vslices, states, decays);
     }
     if (bonus) XRT_REC_DIM(true, true); else XRT_REC_DIM(false, true);
