@@ -473,3 +473,45 @@ def test_small_operations(ops):
 
 def test_the_largest_errors_seen_are_reported():
     print("largest errors against the plain model (max, rms):", {k: [f"{x:.2e}" for x in v] for k, v in WORST.items()})
+
+
+# ---- through the programs a user runs ----------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_replay_of_whole_requests_decoded_tails_and_batches(dtype, models, tmp_path):
+    """`bin/trace_run` as a program of its own on a folder whose config.json leaves the inner widths to the tensors: each
+    request whole, with its last tokens one by one, and in batches of unequal requests that are decoded together."""
+    from test_trace_run_gpu import collect, replay, trace_batches, trace_tail, trace_whole
+    folder, plain, _, _ = models["wide"]
+    vocab = CONFIGS["wide"]["vocab"]
+    lengths = {"a": 40, "b": 7, "c": 100, "d": 65, "e": 1, "f": 90}
+    requests = {n: token_ids(vocab, length, seed=length) for n, length in lengths.items()}
+    want = {n: plain.logits(ids) for n, ids in requests.items()}
+    whole = trace_whole(requests)
+    got_whole = collect(whole, replay(folder, dtype, tmp_path / "whole", whole, 128))
+    tail = trace_tail(requests)
+    got_tail = collect(tail, replay(folder, dtype, tmp_path / "tail", tail, 128))
+    names = list(requests)
+    batches = [{n: requests[n] for n in names[:3]}, {n: requests[n] for n in names[3:]}]
+    batched = trace_batches(batches, lambda n, ids: max(1, len(ids) - 5 - ord(n) % 3))
+    got_batched = collect(batched, replay(folder, dtype, tmp_path / "batched", batched, 256))
+    for n in names:
+        assert_logits(got_whole[n], want[n], dtype, f"trace whole {n}")
+        assert_logits(got_tail[n], want[n], dtype, f"trace tail {n}")
+        assert_logits(got_batched[n], want[n], dtype, f"trace batched {n}")
+
+
+def test_the_command_line_generates_what_the_plain_loop_does(models):
+    import os
+    import subprocess
+    import sys
+    folder, plain, ids, _ = models["mixed"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    prompts = [ids[:5], ids[30:31]]
+    done = subprocess.run([sys.executable, os.path.join(root, "bin", "xrt"), "generate", "--model", folder, "--dtype", "float32",
+                           "--prompt-ids", ";".join(",".join(map(str, p)) for p in prompts), "--max-tokens", "6",
+                           "--temperature", "0", "--repetition-penalty", "1.0", "--stop-ids", ""],
+                          capture_output=True, text=True, timeout=600)
+    assert done.returncode == 0, done.stderr
+    lines = [line for line in done.stdout.splitlines() if line.strip()]
+    assert [[int(t) for t in line.split()] for line in lines] == [P.generate_greedy(plain, p, 6) for p in prompts]

@@ -26,7 +26,8 @@ def replay(folder, dtype, out, steps, max_tokens):
     assert done.returncode == 0, done.stderr[-2000:]
     lines = [line for line in done.stdout.splitlines() if line.startswith("done ")]
     assert lines == [f"done {step['step']}" for step in steps]
-    vocab = json.load(open(os.path.join(folder, "config.json")))["vocab_size"]
+    raw = json.load(open(os.path.join(folder, "config.json")))
+    vocab = raw["vocab_size"] if "vocab_size" in raw else raw["vocab"]
     result = {}
     for step in steps:
         path = os.path.join(str(out), f"{step['step']}.f32")
