@@ -53,15 +53,58 @@ template <typename T> struct alignas(sizeof(T) * 4) Vec4 { T e[4]; };
 // together, and kept in registers between the sum and the scaling (up to CACHED * 1024 elements;
 // the rest of a longer row is read twice). Other rows take the scalar path. The order of the sum
 // depends only on the row length.
-template <typename TW, typename TO>
+//
+// CONV: a step in which every sequence brings one token may let this kernel also do the short convolution over time that
+// reads the normed row (csrc/sequence_state.hip: xrt_short_conv, whose arithmetic this repeats term for term on the normed
+// values as the norm alone would have rounded them): out = conv(normed) (+ normed), and the sequence's kept inputs move on
+// by the normed row. A lane touches only its own channels of its row's sequence.
+struct ConvAfterNorm {
+    const void* w;          // [hidden][taps]
+    int w_dtype, taps, plus_input;
+    float* state;           // [slots][taps - 1][hidden]
+    const int* token_slots; // [rows]: negative: padding, whose row becomes zeros
+};
+
+template <typename TO>
+__device__ __forceinline__ float conv_after_norm(const ConvAfterNorm& conv, float normed, int slot, int c, int hidden) {
+    const float now = to_float(from_float<TO>(normed));
+    float* mine = conv.state + (long)slot * (conv.taps - 1) * hidden + c;
+    const long w_at = (long)c * conv.taps;
+    auto weight = [&](int j) { return conv.w_dtype == XRT_F32 ? ((const float*)conv.w)[w_at + j] : to_float(((const bf16*)conv.w)[w_at + j]); };
+    float y = 0.f;
+    for (int m = 0; m < conv.taps - 1; ++m) {
+        const float kept = mine[(long)m * hidden];
+        y = fmaf(weight(m), kept, y);
+        if (m > 0) mine[(long)(m - 1) * hidden] = kept;
+    }
+    y = fmaf(weight(conv.taps - 1), now, y);
+    if (conv.plus_input) y += now;
+    if (conv.taps >= 2) mine[(long)(conv.taps - 2) * hidden] = now;
+    return y;
+}
+
+template <typename TW, typename TO, bool CONV>
 __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ weight,
                                                       float eps, TO* __restrict__ out,
-                                                      const int* __restrict__ rows, int hidden) {
+                                                      const int* __restrict__ rows, int hidden, const ConvAfterNorm conv) {
     constexpr int CACHED = 8;
     __shared__ float scratch[32];
     const long src = rows ? rows[blockIdx.x] : blockIdx.x;
     const float* row = x + src * hidden;
     TO* dst = out + (long)blockIdx.x * hidden;
+    int slot = 0;
+    if constexpr (CONV) {
+        slot = conv.token_slots[blockIdx.x];
+        if (slot < 0) {
+            for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = from_float<TO>(0.f);
+            return;
+        }
+    }
+    // what is written for channel c, whose normed value is given
+    auto finished = [&](float normed, int c) {
+        if constexpr (CONV) return from_float<TO>(conv_after_norm<TO>(conv, normed, slot, c, hidden));
+        else return from_float<TO>(normed);
+    };
     if (hidden % 4 == 0) {
         const int quads = hidden / 4;
         const float4* row4 = reinterpret_cast<const float4*>(row);
@@ -85,10 +128,10 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
         const float inv_rms = 1.0f / sqrtf(sum / (float)hidden + eps);
         auto emit = [&](int q, const float4& v, const Vec4<TW>& w) {
             Vec4<TO> r;
-            r.e[0] = from_float<TO>((v.x * inv_rms) * to_float(w.e[0]));
-            r.e[1] = from_float<TO>((v.y * inv_rms) * to_float(w.e[1]));
-            r.e[2] = from_float<TO>((v.z * inv_rms) * to_float(w.e[2]));
-            r.e[3] = from_float<TO>((v.w * inv_rms) * to_float(w.e[3]));
+            r.e[0] = finished((v.x * inv_rms) * to_float(w.e[0]), 4 * q);
+            r.e[1] = finished((v.y * inv_rms) * to_float(w.e[1]), 4 * q + 1);
+            r.e[2] = finished((v.z * inv_rms) * to_float(w.e[2]), 4 * q + 2);
+            r.e[3] = finished((v.w * inv_rms) * to_float(w.e[3]), 4 * q + 3);
             *reinterpret_cast<Vec4<TO>*>(dst + 4 * q) = r;
         };
 #pragma unroll
@@ -104,7 +147,7 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
     sum = block_sum(sum, scratch);
     const float inv_rms = 1.0f / sqrtf(sum / (float)hidden + eps);
     for (int i = threadIdx.x; i < hidden; i += blockDim.x)
-        dst[i] = from_float<TO>((row[i] * inv_rms) * to_float(weight[i]));
+        dst[i] = finished((row[i] * inv_rms) * to_float(weight[i]), i);
 }
 
 extern "C" int xrt_embed(const void* table, int table_dtype, const xrt_packing* packing, const int* ids, float* out, int tokens,
@@ -149,12 +192,32 @@ extern "C" int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype,
                 "rmsnorm: unknown dtype weight=%d out=%d", weight_dtype, out_dtype);
     if (n_rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-#define XRT_RMS(TW, TO) rmsnorm_kernel<TW, TO><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, rows, hidden)
+#define XRT_RMS(TW, TO) rmsnorm_kernel<TW, TO, false><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, rows, hidden, ConvAfterNorm{})
     if (weight_dtype == XRT_F32 && out_dtype == XRT_F32) XRT_RMS(float, float);
     else if (weight_dtype == XRT_F32) XRT_RMS(float, bf16);
     else if (out_dtype == XRT_F32) XRT_RMS(bf16, float);
     else XRT_RMS(bf16, bf16);
 #undef XRT_RMS
     XRT_LAUNCH_CHECK("rmsnorm");
+    return 0;
+}
+
+extern "C" int xrt_rmsnorm_conv_step(const float* x, const void* weight, int weight_dtype, float eps, void* out, int out_dtype, int n_rows,
+                                     int hidden, const void* conv_w, int conv_w_dtype, int taps, int plus_input, float* state,
+                                     const int* token_slots, void* stream) {
+    XRT_REQUIRE(n_rows >= 0 && hidden > 0, "rmsnorm_conv_step: bad sizes rows=%d hidden=%d", n_rows, hidden);
+    XRT_REQUIRE((weight_dtype == XRT_F32 || weight_dtype == XRT_BF16) && (out_dtype == XRT_F32 || out_dtype == XRT_BF16) &&
+                (conv_w_dtype == XRT_F32 || conv_w_dtype == XRT_BF16), "rmsnorm_conv_step: unknown dtype");
+    XRT_REQUIRE(x && weight && out && conv_w && token_slots && (state || taps == 1) && taps >= 1, "rmsnorm_conv_step: null operand");
+    if (n_rows == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    const ConvAfterNorm conv{conv_w, conv_w_dtype, taps, plus_input, state, token_slots};
+#define XRT_RMS(TW, TO) rmsnorm_kernel<TW, TO, true><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, nullptr, hidden, conv)
+    if (weight_dtype == XRT_F32 && out_dtype == XRT_F32) XRT_RMS(float, float);
+    else if (weight_dtype == XRT_F32) XRT_RMS(float, bf16);
+    else if (out_dtype == XRT_F32) XRT_RMS(bf16, float);
+    else XRT_RMS(bf16, bf16);
+#undef XRT_RMS
+    XRT_LAUNCH_CHECK("rmsnorm_conv_step");
     return 0;
 }

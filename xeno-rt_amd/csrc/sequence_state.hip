@@ -117,8 +117,11 @@ __global__ void __launch_bounds__(CONV_THREADS) short_conv_kernel(
 constexpr int REC_SEGMENT = 32;           // fewest tokens of a segment
 constexpr int REC_WAVES_WANTED = 4096;    // segments are made until the launch has about this many wavefronts (a few to every SIMD)
 
+constexpr int REC_SPLIT_ROWS = 32;        // rows of the state that a wavefront takes where the rows of a head are split
+
 struct RecurrencePlan {
     int vslices, segment, segments;       // wavefronts per head; tokens per segment; segments of the longest sequence
+    int row_split;                        // wavefronts that share the rows of a head's state (their outputs are added afterwards)
     long raw_floats, state_floats, decay_floats;
 };
 
@@ -130,7 +133,11 @@ RecurrencePlan recurrence_plan(int n_seqs, int max_count, long tokens, int heads
     const long length = (max_count + wanted - 1) / wanted;
     p.segment = (int)max((long)REC_SEGMENT, (length + 15) / 16 * 16);
     p.segments = max(1, (max_count + p.segment - 1) / p.segment);
-    p.raw_floats = tokens * heads * vdim;
+    // A step of few tokens a sequence (a decode step above all) has little to do and much to wait for: the rows of a state
+    // are then dealt to wavefronts of REC_SPLIT_ROWS rows each. The rule looks at the longest run of tokens only, never at
+    // how many sequences there are, so a request's bits do not depend on what else is in the batch.
+    p.row_split = max_count <= REC_SEGMENT ? (dim + REC_SPLIT_ROWS - 1) / REC_SPLIT_ROWS : 1;
+    p.raw_floats = tokens * heads * vdim * p.row_split;
     p.state_floats = p.segments > 1 ? (long)n_seqs * (p.segments + 1) * heads * dim * vdim : 0;
     p.decay_floats = p.segments > 1 ? (long)n_seqs * p.segments * heads * dim : 0;
     return p;
@@ -143,52 +150,59 @@ __device__ __forceinline__ float lane_value(float v, int lane) {
 // What a token brings, across the lanes: channel lane + 64 m in element m. Channels beyond dim read as q = k = 0, decay = 1.
 template <int M>
 struct TokenInputs {
-    float q[M], k[M], d[M], v, bonus_dot;
+    float q[M], k[M], d[M], v;
 };
 
-template <int M, bool BONUS>
-__device__ __forceinline__ void load_token(TokenInputs<M>& in, const xrt_recurrence& a, int dtype, long row, int head, int column, bool owner) {
+// The decay of key channel `at` (head * dim + channel) at the token in `row`.
+__device__ __forceinline__ float decay_of(const xrt_recurrence& a, long row, int head, long at) {
+    if (a.decay_mode == XRT_DECAY_PER_HEAD) return a.decay[head];
+    float z = a.decay[row * (long)a.heads * a.dim + at];
+    if (a.decay_bias != nullptr) z += load_as_float(a.decay_bias, a.decay_bias_dtype, at);
+    if (a.decay_mode == XRT_DECAY_EXP_NEG_EXP) return expf(-expf(z));
+    if (a.decay_mode == XRT_DECAY_SIGMOID_POWER) return expf(-softplus_exact(-z) * a.decay_power);       // sigmoid(z)^power
+    return z;
+}
+
+// rows: the channels row0 .. row0 + rows of the head are this wavefront's
+template <int M>
+__device__ __forceinline__ void load_token(TokenInputs<M>& in, const xrt_recurrence& a, int dtype, long row, int head, int column, bool owner,
+                                           int row0, int rows) {
     const int lane = threadIdx.x;
-    float dot = 0.f;
 #pragma unroll
     for (int m = 0; m < M; ++m) {
         const int i = lane + XRT_WAVE * m;
         in.q[m] = 0.f; in.k[m] = 0.f; in.d[m] = 1.f;
-        if (i < a.dim) {
-            const long at = (long)head * a.dim + i;
+        if (i < rows) {
+            const long at = (long)head * a.dim + row0 + i;
             in.q[m] = load_as_float(a.q, dtype, row * a.q_stride + at) * a.q_scale;
             in.k[m] = load_as_float(a.k, dtype, row * a.k_stride + at) * a.k_scale;
-            if (a.decay_mode == XRT_DECAY_PER_HEAD) {
-                in.d[m] = a.decay[head];
-            } else {
-                float z = a.decay[row * (long)a.heads * a.dim + at];
-                if (a.decay_bias != nullptr) z += load_as_float(a.decay_bias, a.decay_bias_dtype, at);
-                if (a.decay_mode == XRT_DECAY_EXP_NEG_EXP) in.d[m] = expf(-expf(z));
-                else if (a.decay_mode == XRT_DECAY_SIGMOID_POWER) in.d[m] = expf(-softplus_exact(-z) * a.decay_power);   // sigmoid(z)^power
-                else in.d[m] = z;
-            }
-            if constexpr (BONUS) dot = fmaf(load_as_float(a.bonus, a.bonus_dtype, at) * in.k[m], in.q[m], dot);
+            in.d[m] = decay_of(a, row, head, at);
         }
     }
     in.v = owner ? load_as_float(a.v, dtype, row * a.v_stride + (long)head * a.vdim + column) : 0.f;
-    in.bonus_dot = BONUS ? wave_sum(dot) : 0.f;            // sum over the channels of bonus * k * q: what the token's own k v^T adds to its output
 }
 
-// grid (sequences, heads * vslices, segments), one wavefront each.
+// grid (sequences, heads * vslices * row_split, segments), one wavefront each. With row_split > 1 (one segment only) a wavefront
+// has DIM rows of the state, and what it writes to raw, into a part of its own, is its rows' share of the outputs. With a bonus
+// the token is read before it enters the state; what its own k v^T adds to its output is left to the pass over the raw outputs.
 // FINAL false: a segment from empty hands, no outputs: its L to states[seq][segment], its P to decays[seq][segment].
 // FINAL true: from the state at the segment's beginning (the cache's for a sequence in one segment, else states[...]: entry
 // `segments` for the first segment, entry c - 1 for segment c), raw outputs to raw [tokens][heads * vdim]; a sequence's last
 // segment leaves the state in the cache.
 template <int DIM, bool BONUS, bool FINAL>
 __global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurrence a, int dtype, const int* __restrict__ seq_offsets,
-                                                             const int* __restrict__ seq_slots, int segment, int segments, int vslices,
-                                                             float* __restrict__ states, float* __restrict__ decays, float* __restrict__ raw) {
+                                                             const int* __restrict__ seq_slots, int segment, int segments, int vslices, int row_split,
+                                                             float* __restrict__ states, float* __restrict__ decays, float* __restrict__ raw_all,
+                                                             long tokens) {
     constexpr int M = (DIM + XRT_WAVE - 1) / XRT_WAVE;
-    const int seq = blockIdx.x, head = blockIdx.y / vslices, vslice = blockIdx.y % vslices, lane = threadIdx.x;
+    const int seq = blockIdx.x, part = blockIdx.y % row_split, head = blockIdx.y / row_split / vslices, vslice = blockIdx.y / row_split % vslices;
+    const int lane = threadIdx.x;
     const int begin = seq_offsets[seq], count = seq_offsets[seq + 1] - begin, slot = seq_slots[seq];
     const int first = blockIdx.z * segment, last = min(count, first + segment);
     if (first >= count) return;
-    const int dim = a.dim, vdim = a.vdim, heads = a.heads;
+    const int vdim = a.vdim, heads = a.heads;
+    const int row0 = row_split > 1 ? part * DIM : 0, dim = min(row_split > 1 ? DIM : a.dim, a.dim - row0);     // this wavefront's rows
+    float* raw = raw_all + (long)part * tokens * heads * vdim;
     const int column = vslice * XRT_WAVE + lane;
     const bool owner = column < vdim;
     const bool ends_sequence = last == count, whole = count <= segment;
@@ -198,8 +212,8 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurren
             for (int t = first; t < last; ++t) raw[(long)(begin + t) * heads * vdim + (long)head * vdim + column] = 0.f;
         return;
     }
-    const long per_head = (long)dim * vdim;
-    float* cached = a.state + ((long)slot * heads + head) * per_head + column;
+    const long per_head = (long)a.dim * vdim;
+    float* cached = a.state + ((long)slot * heads + head) * per_head + (long)row0 * vdim + column;
     float* at_segment = states + (((long)seq * (segments + 1) + blockIdx.z) * heads + head) * per_head + column;
     float S[DIM];
     if (FINAL) {
@@ -216,9 +230,9 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurren
     for (int m = 0; m < M; ++m) product[m] = 1.f;
 
     TokenInputs<M> now, next;
-    load_token<M, BONUS>(now, a, dtype, begin + first, head, column, owner);
+    load_token<M>(now, a, dtype, begin + first, head, column, owner, row0, dim);
     for (int t = first; t < last; ++t) {
-        if (t + 1 < last) load_token<M, BONUS>(next, a, dtype, begin + t + 1, head, column, owner);
+        if (t + 1 < last) load_token<M>(next, a, dtype, begin + t + 1, head, column, owner, row0, dim);
         float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int g = 0; g < DIM / 16; ++g) {
@@ -249,7 +263,6 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurren
         }
         if constexpr (FINAL) {
             float out = (o[0] + o[1]) + (o[2] + o[3]);
-            if constexpr (BONUS) out = fmaf(now.bonus_dot, now.v, out);
             if (owner) raw[(long)(begin + t) * heads * vdim + (long)head * vdim + column] = out;
         } else {
 #pragma unroll
@@ -273,7 +286,7 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_kernel(const xrt_recurren
 #pragma unroll
             for (int m = 0; m < M; ++m)
                 if (lane + XRT_WAVE * m < dim)
-                    decays[(((long)seq * segments + blockIdx.z) * heads + head) * dim + lane + XRT_WAVE * m] = product[m];
+                    decays[(((long)seq * segments + blockIdx.z) * heads + head) * a.dim + lane + XRT_WAVE * m] = product[m];
         }
     }
 }
@@ -313,7 +326,7 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_combine_kernel(const xrt_
 
 // The heads' raw outputs of one token: norm over vdim, weight, gate. A wavefront per (token, head).
 __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_recurrence a, int dtype, const float* __restrict__ raw,
-                                                                    const int* __restrict__ token_slots) {
+                                                                    const int* __restrict__ token_slots, int row_split, long tokens) {
     const long row = blockIdx.x;
     const int head = blockIdx.y, lane = threadIdx.x, vdim = a.vdim;
     const long out_at = row * a.heads * vdim + (long)head * vdim;
@@ -321,14 +334,31 @@ __global__ void __launch_bounds__(XRT_WAVE) recurrence_finish_kernel(const xrt_r
         for (int c = lane; c < vdim; c += XRT_WAVE) store_from_float(a.out, dtype, out_at + c, 0.f);
         return;
     }
+    // what the token's own k v^T adds to its output where it is read with a bonus: v * sum over the channels of bonus * k * q
+    float bonus_dot = 0.f;
+    if (a.bonus != nullptr) {
+        for (int i = lane; i < a.dim; i += XRT_WAVE) {
+            const long at = (long)head * a.dim + i;
+            const float k = load_as_float(a.k, dtype, row * a.k_stride + at) * a.k_scale, q = load_as_float(a.q, dtype, row * a.q_stride + at) * a.q_scale;
+            bonus_dot = fmaf(load_as_float(a.bonus, a.bonus_dtype, at) * k, q, bonus_dot);
+        }
+        bonus_dot = wave_sum(bonus_dot);
+    }
+    // the parts of the wavefronts that shared the state's rows, in their order
+    auto whole = [&](int c) {
+        float sum = raw[out_at + c];
+        for (int part = 1; part < row_split; ++part) sum += raw[(long)part * tokens * a.heads * vdim + out_at + c];
+        if (a.bonus != nullptr) sum = fmaf(bonus_dot, load_as_float(a.v, dtype, row * a.v_stride + (long)head * vdim + c), sum);
+        return sum;
+    };
     float inv = 1.f;
     if (a.norm) {
         float squares = 0.f;
-        for (int c = lane; c < vdim; c += XRT_WAVE) squares = fmaf(raw[out_at + c], raw[out_at + c], squares);
+        for (int c = lane; c < vdim; c += XRT_WAVE) { const float o = whole(c); squares = fmaf(o, o, squares); }
         inv = 1.0f / sqrtf(wave_sum(squares) / (float)vdim + a.eps);
     }
     for (int c = lane; c < vdim; c += XRT_WAVE) {
-        float value = raw[out_at + c] * inv;
+        float value = whole(c) * inv;
         if (a.norm_weight != nullptr)
             value *= load_as_float(a.norm_weight, a.norm_weight_dtype, a.norm_weight_per_head ? (long)head * vdim + c : c);
         if (a.gate != nullptr) {
@@ -471,12 +501,13 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
     float* states = raw + p.raw_floats;
     float* decays = states + p.state_floats;
     const bool bonus = a.bonus != nullptr;
-    const dim3 grid(n_seqs, a.heads * p.vslices, p.segments);
+    XRT_REQUIRE((long)a.heads * p.vslices * p.row_split <= 65535, "linear_recurrence: too many heads for one launch");
+    const dim3 grid(n_seqs, a.heads * p.vslices * p.row_split, p.segments);
 #define XRT_REC(DIM_, BONUS_, FINAL_) recurrence_kernel<DIM_, BONUS_, FINAL_><<<grid, XRT_WAVE, 0, s>>>(a, dtype, seq_offsets, seq_slots, \
-        p.segment, p.segments, p.vslices, states, decays, raw)
+        p.segment, p.segments, p.vslices, p.row_split, states, decays, raw, tokens)
 #define XRT_REC_DIM(BONUS_, FINAL_)                                                                \
     do {                                                                                           \
-        if (a.dim <= 32) XRT_REC(32, BONUS_, FINAL_); else if (a.dim <= 64) XRT_REC(64, BONUS_, FINAL_); \
+        if (a.dim <= 32 || p.row_split > 1) XRT_REC(REC_SPLIT_ROWS, BONUS_, FINAL_); else if (a.dim <= 64) XRT_REC(64, BONUS_, FINAL_); \
         else if (a.dim <= 128) XRT_REC(128, BONUS_, FINAL_); else XRT_REC(256, BONUS_, FINAL_);    \
     } while (0)
     if (p.segments > 1) {
@@ -487,7 +518,7 @@ extern "C" int xrt_linear_recurrence(const xrt_recurrence* args, int dtype, cons
     if (bonus) XRT_REC_DIM(true, true); else XRT_REC_DIM(false, true);
 #undef XRT_REC_DIM
 #undef XRT_REC
-    recurrence_finish_kernel<<<dim3((unsigned)tokens, a.heads), XRT_WAVE, 0, s>>>(a, dtype, raw, token_slots);
+    recurrence_finish_kernel<<<dim3((unsigned)tokens, a.heads), XRT_WAVE, 0, s>>>(a, dtype, raw, token_slots, p.row_split, tokens);
     XRT_LAUNCH_CHECK("linear_recurrence");
     return 0;
 }

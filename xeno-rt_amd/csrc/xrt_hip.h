@@ -63,6 +63,12 @@ int xrt_add(float* residual, const void* delta, int delta_dtype, long count, voi
 int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype, float eps, void* out, int out_dtype,
                 const int* rows, int n_rows, int hidden, void* stream);
 
+// xrt_rmsnorm of every row, then xrt_short_conv of the normed rows (plain, or plus the input), for a step in which row r is the
+// one new token of the sequence in slot token_slots[r] (negative: padding, the row becomes zeros): one kernel, the same bits.
+int xrt_rmsnorm_conv_step(const float* x, const void* weight, int weight_dtype, float eps, void* out, int out_dtype, int n_rows,
+                          int hidden, const void* conv_w, int conv_w_dtype, int taps, int plus_input, float* state,
+                          const int* token_slots, void* stream);
+
 // out[m, n] (+)= sum_k a[m, k] * w[n, k]   (mode 0 store, 1 accumulate into float32 out,
 // 2 gated: out[m, n] = act(a.w[n]) * (a.w[n + N]) with w of 2N rows; the activation's code rides above the
 // mode's low byte, XRT_GATED(XRT_ACT_SILU) == 2: silu(z) = z / (1 + exp(-z)) is the one that exists)

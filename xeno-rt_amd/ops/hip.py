@@ -181,7 +181,7 @@ class HipOps:
                      "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits", "xrt_block_tokens",
                      "xrt_attention_finishes_qkv", "xrt_attention_finishing", "xrt_rope_table", "xrt_short_conv",
                      "xrt_linear_recurrence", "xrt_add_normed", "xrt_activation", "xrt_rows_add", "xrt_kv_store",
-                     "xrt_attention_general"):
+                     "xrt_attention_general", "xrt_rmsnorm_conv_step"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -564,6 +564,23 @@ class HipOps:
         self._check(self.lib.xrt_short_conv(_ptr(x), _code(x), ctypes.c_long(tokens), ctypes.c_long(stride), channels, _ptr(w), _code(w), taps,
                                             n_out, CONV_MODES[mode], _ptr(state), offsets, slots, n, int(batch.max_count), _ptr(out),
                                             self._stream(x)))
+
+    def rmsnorm_conv_step(self, x, weight, eps, conv_w, state, batch, out, plus_input=False):
+        """`rmsnorm` of the rows of x, then `short_conv` of the normed rows (plain or plus the input), in one kernel and to the
+        same bits: for a step in which every sequence brings exactly one token."""
+        tokens, hidden = x.shape
+        taps = conv_w.shape[-1]
+        if int(batch.max_count) != 1 or int(batch.n_tokens) != tokens:
+            raise KernelError("rmsnorm_conv_step: a step in which every sequence brings one token")
+        self._require(x, "rmsnorm_conv_step x", torch.float32)
+        self._require(weight, "rmsnorm_conv_step weight", None, (hidden,), x)
+        self._require(conv_w, "rmsnorm_conv_step conv_w", None, (hidden, taps), x)
+        self._require(state, "rmsnorm_conv_step state", torch.float32, (state.shape[0], taps - 1, hidden), x)
+        self._require(out, "rmsnorm_conv_step out", None, (tokens, hidden), x)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), x)
+        self._check(self.lib.xrt_rmsnorm_conv_step(_ptr(x), _ptr(weight), _code(weight), ctypes.c_float(eps), _ptr(out), _code(out), tokens,
+                                                   hidden, _ptr(conv_w), _code(conv_w), taps, int(bool(plus_input)), _ptr(state),
+                                                   _ptr(batch.slots), self._stream(x)))
 
     def linear_recurrence(self, q, k, v, state, batch, out, heads, dim, vdim, decay, decay_mode="per_head", decay_bias=None,
                           decay_power=1.0, q_scale=1.0, k_scale=1.0, bonus=None, norm_eps=None, norm_weight=None, gate=None,

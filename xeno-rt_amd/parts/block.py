@@ -57,17 +57,21 @@ class PreNormBlock(Block):
     def first_norm(self):
         return self.mixer_norm
 
+    @staticmethod
+    def _read(x, norm, transform, batch, cache):
+        """What a sublayer reads: the normed rows, through the sublayer's input transform if it has one (which may do the
+        norm's work as well: `forward_normed`)."""
+        if transform is None:
+            return norm.forward(x)
+        if hasattr(transform, "forward_normed"):
+            return transform.forward_normed(x, norm, batch, cache)
+        return transform.forward(norm.forward(x), batch, cache)
+
     def forward(self, x, batch, cache, h=None, then=None):
         if not self.passes_norms:
-            h = self.mixer_norm.forward(x)
-            if self.mixer_input is not None:
-                h = self.mixer_input.forward(h, batch, cache)
-            self.mixer.forward(h, batch, cache, x)
+            self.mixer.forward(self._read(x, self.mixer_norm, self.mixer_input, batch, cache), batch, cache, x)
             if self.feed_forward is not None:
-                h = self.feed_forward_norm.forward(x)
-                if self.feed_forward_input is not None:
-                    h = self.feed_forward_input.forward(h, batch, cache)
-                self.feed_forward.forward(h, batch, x)
+                self.feed_forward.forward(self._read(x, self.feed_forward_norm, self.feed_forward_input, batch, cache), batch, x)
             return None
         if h is None:
             h = self.mixer_norm.forward(x)

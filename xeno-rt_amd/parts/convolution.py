@@ -45,6 +45,20 @@ class ShortConvolution(Part):
         return out
 
 
+    def forward_normed(self, x: torch.Tensor, norm, batch, cache) -> torch.Tensor:
+        """This convolution of norm(x). Where every sequence brings one token and the norm is a plain RMSNorm over whole
+        rows, one kernel does both (to the same bits as the two would)."""
+        rt = self.runtime
+        scale = norm.row_scale()
+        fused = getattr(rt.ops, "rmsnorm_conv_step", None)
+        if (fused is None or scale is None or len(self.names) != 1 or int(batch.max_count) != 1
+                or int(batch.n_tokens) != int(batch.n_sequences) or x.shape[1] != self.channels):
+            return self.forward(norm.forward(x), batch, cache)
+        out = rt.empty((x.shape[0], self.channels))
+        fused(x, scale[0], scale[1], self.weight, cache.states[self.state_name], batch, out, plus_input=self.plus_input)
+        return out
+
+
 class TokenShift(Part):
     """For each of several readers its own mix of a token and the one before it: u + (u[t - 1] - u) * mu, with
     mu [channels] per reader and zeros before the sequence's start. Returns [readers, tokens, channels]."""
