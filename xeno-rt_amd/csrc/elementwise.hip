@@ -83,6 +83,55 @@ __device__ __forceinline__ float conv_after_norm(const ConvAfterNorm& conv, floa
     return y;
 }
 
+// The same for four neighbouring channels 4 q .. 4 q + 3 at once (hidden a multiple of 4): everything is fetched, sixteen bytes
+// a load, before anything is written, so that the loads are in flight together.
+constexpr int CONV_AFTER_NORM_MOST_TAPS = 16;
+
+template <typename TO>
+__device__ __forceinline__ void conv_after_norm4(const ConvAfterNorm& conv, float (&normed)[4], int slot, int q, int hidden) {
+    float4* mine = reinterpret_cast<float4*>(conv.state + (long)slot * (conv.taps - 1) * hidden) + q;      // row m: + m * hidden / 4
+    const int quads = hidden / 4, taps = conv.taps;
+    float4 kept[CONV_AFTER_NORM_MOST_TAPS - 1];
+    float w[4][CONV_AFTER_NORM_MOST_TAPS];
+#pragma unroll
+    for (int m = 0; m < CONV_AFTER_NORM_MOST_TAPS - 1; ++m)
+        if (m < taps - 1) kept[m] = mine[(long)m * quads];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int j = 0; j < CONV_AFTER_NORM_MOST_TAPS; ++j)
+            if (j < taps) {
+                const long at = ((long)4 * q + e) * taps + j;
+                w[e][j] = conv.w_dtype == XRT_F32 ? ((const float*)conv.w)[at] : to_float(((const bf16*)conv.w)[at]);
+            }
+    float now[4], y[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) now[e] = to_float(from_float<TO>(normed[e]));
+#pragma unroll
+    for (int m = 0; m < CONV_AFTER_NORM_MOST_TAPS - 1; ++m)
+        if (m < taps - 1) {
+            y[0] = fmaf(w[0][m], kept[m].x, y[0]);
+            y[1] = fmaf(w[1][m], kept[m].y, y[1]);
+            y[2] = fmaf(w[2][m], kept[m].z, y[2]);
+            y[3] = fmaf(w[3][m], kept[m].w, y[3]);
+        }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float last = 0.f;
+#pragma unroll
+        for (int j = 0; j < CONV_AFTER_NORM_MOST_TAPS; ++j)
+            if (j == taps - 1) last = w[e][j];
+        y[e] = fmaf(last, now[e], y[e]);
+        if (conv.plus_input) y[e] += now[e];
+    }
+#pragma unroll
+    for (int m = 1; m < CONV_AFTER_NORM_MOST_TAPS - 1; ++m)
+        if (m < taps - 1) mine[(long)(m - 1) * quads] = kept[m];
+    if (taps >= 2) mine[(long)(taps - 2) * quads] = make_float4(now[0], now[1], now[2], now[3]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) normed[e] = y[e];
+}
+
 template <typename TW, typename TO, bool CONV>
 __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ weight,
                                                       float eps, TO* __restrict__ out,
@@ -128,10 +177,11 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
         const float inv_rms = 1.0f / sqrtf(sum / (float)hidden + eps);
         auto emit = [&](int q, const float4& v, const Vec4<TW>& w) {
             Vec4<TO> r;
-            r.e[0] = finished((v.x * inv_rms) * to_float(w.e[0]), 4 * q);
-            r.e[1] = finished((v.y * inv_rms) * to_float(w.e[1]), 4 * q + 1);
-            r.e[2] = finished((v.z * inv_rms) * to_float(w.e[2]), 4 * q + 2);
-            r.e[3] = finished((v.w * inv_rms) * to_float(w.e[3]), 4 * q + 3);
+            float four[4] = {(v.x * inv_rms) * to_float(w.e[0]), (v.y * inv_rms) * to_float(w.e[1]),
+                             (v.z * inv_rms) * to_float(w.e[2]), (v.w * inv_rms) * to_float(w.e[3])};
+            if constexpr (CONV) conv_after_norm4<TO>(conv, four, slot, q, hidden);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r.e[e] = from_float<TO>(four[e]);
             *reinterpret_cast<Vec4<TO>*>(dst + 4 * q) = r;
         };
 #pragma unroll
@@ -209,6 +259,7 @@ extern "C" int xrt_rmsnorm_conv_step(const float* x, const void* weight, int wei
     XRT_REQUIRE((weight_dtype == XRT_F32 || weight_dtype == XRT_BF16) && (out_dtype == XRT_F32 || out_dtype == XRT_BF16) &&
                 (conv_w_dtype == XRT_F32 || conv_w_dtype == XRT_BF16), "rmsnorm_conv_step: unknown dtype");
     XRT_REQUIRE(x && weight && out && conv_w && token_slots && (state || taps == 1) && taps >= 1, "rmsnorm_conv_step: null operand");
+    XRT_REQUIRE(taps <= CONV_AFTER_NORM_MOST_TAPS, "rmsnorm_conv_step: %d taps, up to %d are served", taps, CONV_AFTER_NORM_MOST_TAPS);
     if (n_rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const ConvAfterNorm conv{conv_w, conv_w_dtype, taps, plus_input, state, token_slots};

@@ -29,7 +29,7 @@ __device__ __forceinline__ float softplus_exact(float z) { return fmaxf(z, 0.f) 
 
 // ---- short convolution -----------------------------------------------------------------------------------------
 
-constexpr int CONV_MAX_TAPS = 8;
+constexpr int CONV_MAX_TAPS = 16;
 constexpr int CONV_SEGMENT = 16;          // tokens of a sequence that one workgroup walks
 constexpr int CONV_THREADS = 256;         // channels of a workgroup
 
