@@ -67,6 +67,7 @@ struct ConvAfterNorm {
 
 template <typename TO>
 __device__ __forceinline__ float conv_after_norm(const ConvAfterNorm& conv, float normed, int slot, int c, int hidden) {
+#pragma clang fp contract(off)      // (only the products and sums written as fmaf are fused: the same in every kernel that does this convolution)
     const float now = to_float(from_float<TO>(normed));
     float* mine = conv.state + (long)slot * (conv.taps - 1) * hidden + c;
     const long w_at = (long)c * conv.taps;
@@ -83,60 +84,53 @@ __device__ __forceinline__ float conv_after_norm(const ConvAfterNorm& conv, floa
     return y;
 }
 
-// The same for four neighbouring channels 4 q .. 4 q + 3 at once (hidden a multiple of 4): everything is fetched, sixteen bytes
-// a load, before anything is written, so that the loads are in flight together.
-constexpr int CONV_AFTER_NORM_MOST_TAPS = 16;
+// The same for four neighbouring channels 4 q .. 4 q + 3 at once (hidden a multiple of 4), the number of taps known when the
+// kernel is compiled: everything is fetched, sixteen bytes a load, before anything is written, so that the loads are in flight together.
+constexpr int CONV_AFTER_NORM_MOST_TAPS = 8;
 
-template <typename TO>
+template <typename TO, int TAPS>
 __device__ __forceinline__ void conv_after_norm4(const ConvAfterNorm& conv, float (&normed)[4], int slot, int q, int hidden) {
-    float4* mine = reinterpret_cast<float4*>(conv.state + (long)slot * (conv.taps - 1) * hidden) + q;      // row m: + m * hidden / 4
-    const int quads = hidden / 4, taps = conv.taps;
-    float4 kept[CONV_AFTER_NORM_MOST_TAPS - 1];
-    float w[4][CONV_AFTER_NORM_MOST_TAPS];
+#pragma clang fp contract(off)      // (only the products and sums written as fmaf are fused: the same in every kernel that does this convolution)
+    float4* mine = reinterpret_cast<float4*>(conv.state + (long)slot * (TAPS - 1) * hidden) + q;      // row m: + m * hidden / 4
+    const int quads = hidden / 4;
+    float4 kept[TAPS > 1 ? TAPS - 1 : 1];
+    float w[4 * TAPS];                                      // of channel 4 q + e: w[e * TAPS ..]
 #pragma unroll
-    for (int m = 0; m < CONV_AFTER_NORM_MOST_TAPS - 1; ++m)
-        if (m < taps - 1) kept[m] = mine[(long)m * quads];
+    for (int m = 0; m < TAPS - 1; ++m) kept[m] = mine[(long)m * quads];
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-#pragma unroll
-        for (int j = 0; j < CONV_AFTER_NORM_MOST_TAPS; ++j)
-            if (j < taps) {
-                const long at = ((long)4 * q + e) * taps + j;
-                w[e][j] = conv.w_dtype == XRT_F32 ? ((const float*)conv.w)[at] : to_float(((const bf16*)conv.w)[at]);
-            }
+    for (int i = 0; i < 4 * TAPS; ++i) {
+        const long at = (long)4 * q * TAPS + i;
+        w[i] = conv.w_dtype == XRT_F32 ? ((const float*)conv.w)[at] : to_float(((const bf16*)conv.w)[at]);
+    }
     float now[4], y[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int e = 0; e < 4; ++e) now[e] = to_float(from_float<TO>(normed[e]));
 #pragma unroll
-    for (int m = 0; m < CONV_AFTER_NORM_MOST_TAPS - 1; ++m)
-        if (m < taps - 1) {
-            y[0] = fmaf(w[0][m], kept[m].x, y[0]);
-            y[1] = fmaf(w[1][m], kept[m].y, y[1]);
-            y[2] = fmaf(w[2][m], kept[m].z, y[2]);
-            y[3] = fmaf(w[3][m], kept[m].w, y[3]);
-        }
+    for (int m = 0; m < TAPS - 1; ++m) {
+        y[0] = fmaf(w[0 * TAPS + m], kept[m].x, y[0]);
+        y[1] = fmaf(w[1 * TAPS + m], kept[m].y, y[1]);
+        y[2] = fmaf(w[2 * TAPS + m], kept[m].z, y[2]);
+        y[3] = fmaf(w[3 * TAPS + m], kept[m].w, y[3]);
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        float last = 0.f;
-#pragma unroll
-        for (int j = 0; j < CONV_AFTER_NORM_MOST_TAPS; ++j)
-            if (j == taps - 1) last = w[e][j];
-        y[e] = fmaf(last, now[e], y[e]);
+        y[e] = fmaf(w[e * TAPS + TAPS - 1], now[e], y[e]);
         if (conv.plus_input) y[e] += now[e];
     }
 #pragma unroll
-    for (int m = 1; m < CONV_AFTER_NORM_MOST_TAPS - 1; ++m)
-        if (m < taps - 1) mine[(long)(m - 1) * quads] = kept[m];
-    if (taps >= 2) mine[(long)(taps - 2) * quads] = make_float4(now[0], now[1], now[2], now[3]);
+    for (int m = 1; m < TAPS - 1; ++m) mine[(long)(m - 1) * quads] = kept[m];
+    if constexpr (TAPS >= 2) mine[(long)(TAPS - 2) * quads] = make_float4(now[0], now[1], now[2], now[3]);
 #pragma unroll
     for (int e = 0; e < 4; ++e) normed[e] = y[e];
 }
 
-template <typename TW, typename TO, bool CONV>
+// TAPS: 0 for the norm alone, else the taps of the convolution that follows it
+template <typename TW, typename TO, int TAPS>
 __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ weight,
                                                       float eps, TO* __restrict__ out,
                                                       const int* __restrict__ rows, int hidden, const ConvAfterNorm conv) {
     constexpr int CACHED = 8;
+    constexpr bool CONV = TAPS > 0;
     __shared__ float scratch[32];
     const long src = rows ? rows[blockIdx.x] : blockIdx.x;
     const float* row = x + src * hidden;
@@ -179,7 +173,7 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
             Vec4<TO> r;
             float four[4] = {(v.x * inv_rms) * to_float(w.e[0]), (v.y * inv_rms) * to_float(w.e[1]),
                              (v.z * inv_rms) * to_float(w.e[2]), (v.w * inv_rms) * to_float(w.e[3])};
-            if constexpr (CONV) conv_after_norm4<TO>(conv, four, slot, q, hidden);
+            if constexpr (CONV) conv_after_norm4<TO, TAPS>(conv, four, slot, q, hidden);
 #pragma unroll
             for (int e = 0; e < 4; ++e) r.e[e] = from_float<TO>(four[e]);
             *reinterpret_cast<Vec4<TO>*>(dst + 4 * q) = r;
@@ -242,7 +236,7 @@ extern "C" int xrt_rmsnorm(const float* x, const void* weight, int weight_dtype,
                 "rmsnorm: unknown dtype weight=%d out=%d", weight_dtype, out_dtype);
     if (n_rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-#define XRT_RMS(TW, TO) rmsnorm_kernel<TW, TO, false><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, rows, hidden, ConvAfterNorm{})
+#define XRT_RMS(TW, TO) rmsnorm_kernel<TW, TO, 0><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, rows, hidden, ConvAfterNorm{})
     if (weight_dtype == XRT_F32 && out_dtype == XRT_F32) XRT_RMS(float, float);
     else if (weight_dtype == XRT_F32) XRT_RMS(float, bf16);
     else if (out_dtype == XRT_F32) XRT_RMS(bf16, float);
@@ -263,11 +257,25 @@ extern "C" int xrt_rmsnorm_conv_step(const float* x, const void* weight, int wei
     if (n_rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     const ConvAfterNorm conv{conv_w, conv_w_dtype, taps, plus_input, state, token_slots};
-#define XRT_RMS(TW, TO) rmsnorm_kernel<TW, TO, true><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, nullptr, hidden, conv)
-    if (weight_dtype == XRT_F32 && out_dtype == XRT_F32) XRT_RMS(float, float);
-    else if (weight_dtype == XRT_F32) XRT_RMS(float, bf16);
-    else if (out_dtype == XRT_F32) XRT_RMS(bf16, float);
-    else XRT_RMS(bf16, bf16);
+#define XRT_RMS(TW, TO, TAPS_) rmsnorm_kernel<TW, TO, TAPS_><<<n_rows, 256, 0, s>>>(x, (const TW*)weight, eps, (TO*)out, nullptr, hidden, conv)
+#define XRT_RMS_TYPES(TAPS_)                                                                 \
+    do {                                                                                     \
+        if (weight_dtype == XRT_F32 && out_dtype == XRT_F32) XRT_RMS(float, float, TAPS_);   \
+        else if (weight_dtype == XRT_F32) XRT_RMS(float, bf16, TAPS_);                       \
+        else if (out_dtype == XRT_F32) XRT_RMS(bf16, float, TAPS_);                          \
+        else XRT_RMS(bf16, bf16, TAPS_);                                                     \
+    } while (0)
+    switch (taps) {
+        case 1: XRT_RMS_TYPES(1); break;
+        case 2: XRT_RMS_TYPES(2); break;
+        case 3: XRT_RMS_TYPES(3); break;
+        case 4: XRT_RMS_TYPES(4); break;
+        case 5: XRT_RMS_TYPES(5); break;
+        case 6: XRT_RMS_TYPES(6); break;
+        case 7: XRT_RMS_TYPES(7); break;
+        default: XRT_RMS_TYPES(8); break;
+    }
+#undef XRT_RMS_TYPES
 #undef XRT_RMS
     XRT_LAUNCH_CHECK("rmsnorm_conv_step");
     return 0;

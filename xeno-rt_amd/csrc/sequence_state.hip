@@ -48,6 +48,7 @@ __global__ void __launch_bounds__(CONV_THREADS) short_conv_kernel(
     const T* __restrict__ x, long x_stride, int channels, const void* __restrict__ w, int w_dtype, int taps, int n_out, int mode,
     float* __restrict__ state, const int* __restrict__ seq_offsets, const int* __restrict__ seq_slots, T* __restrict__ out,
     long tokens, int phase) {
+#pragma clang fp contract(off)      // (only the products and sums written as fmaf are fused: the same in every kernel that does this convolution)
     const int seq = blockIdx.x, c = blockIdx.z * CONV_THREADS + threadIdx.x;
     if (c >= channels) return;
     const int begin = seq_offsets[seq], count = seq_offsets[seq + 1] - begin, slot = seq_slots[seq];

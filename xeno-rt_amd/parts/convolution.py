@@ -52,7 +52,7 @@ class ShortConvolution(Part):
         scale = norm.row_scale()
         fused = getattr(rt.ops, "rmsnorm_conv_step", None)
         if (fused is None or scale is None or len(self.names) != 1 or int(batch.max_count) != 1
-                or int(batch.n_tokens) != int(batch.n_sequences) or x.shape[1] != self.channels):
+                or int(batch.n_tokens) != int(batch.n_sequences) or x.shape[1] != self.channels or self.taps > 8):
             return self.forward(norm.forward(x), batch, cache)
         out = rt.empty((x.shape[0], self.channels))
         fused(x, scale[0], scale[1], self.weight, cache.states[self.state_name], batch, out, plus_input=self.plus_input)
