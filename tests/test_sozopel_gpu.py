@@ -27,7 +27,9 @@ LENGTH = {"mixed": 150, "wide": 140, "one_tap": 90}
 # cancels (the first tokens of a sequence, whose state holds one or two keys), the rounding of that sum is scaled up
 # with it, so single logits, and the root mean square over a sequence of one or two tokens, differ by more than the
 # sums' own rounding (largest seen: 2.8e-5 and 8.8e-6, on a one-token sequence).
-LIMITS = {"float32": dict(max=1e-4, rms=2e-5), "bfloat16": dict(max=1e-1, rms=2.5e-2)}
+# In bfloat16 the same happens to the rounding of q and k themselves: single logits of the configurations drawn at random (width
+# 136, weights of deviation 0.2) are off by up to 1.3e-1 where the root mean square is 1e-2.
+LIMITS = {"float32": dict(max=1e-4, rms=2e-5), "bfloat16": dict(max=1.5e-1, rms=2.5e-2)}
 WORST = {}
 
 
@@ -515,3 +517,49 @@ def test_the_command_line_generates_what_the_plain_loop_does(models):
     assert done.returncode == 0, done.stderr
     lines = [line for line in done.stdout.splitlines() if line.strip()]
     assert [[int(t) for t in line.split()] for line in lines] == [P.generate_greedy(plain, p, 6) for p in prompts]
+
+
+# ---- configurations drawn at random: other sizes, orders and constants than any above -----------------------------------
+
+def random_configuration(seed):
+    import random
+    r = random.Random(seed)
+    width = r.choice([24, 40, 72, 96, 136])
+    layers = []
+    for _ in range(r.randint(2, 5)):
+        kind = r.choice(["retention", "wkv", "parallel"])
+        if kind == "retention":
+            heads = r.randint(1, 4)
+            mixer = {"heads": heads, "dim": r.choice([4, 12, 20, 32, 48]), "vdim": r.choice([8, 20, 40, 72]),
+                     "decay": [round(1.0 - 2.0 ** -r.randint(1, 9), 6) for _ in range(heads)]}
+        elif kind == "wkv":
+            mixer = {"heads": r.randint(1, 5), "dim": r.choice([8, 16, 24, 40, 64]), "rank": r.choice([3, 8, 12])}
+        else:
+            kv_heads = r.randint(1, 3)
+            mixer = {"left": {"heads": kv_heads * r.randint(1, 3), "kv_heads": kv_heads, "dim": r.choice([6, 16, 20, 32, 64]),
+                              "vdim": r.choice([4, 16, 24, 32, 96]), "conv": r.randint(1, 6), "mask": {"size": r.choice([1, 2, 9, 40, 64, 65, 300])},
+                              "scale": r.choice([0.1, 0.25, 0.5])},
+                     "right": {"heads": r.randint(1, 3), "dim": r.choice([8, 24, 32, 72]), "vdim": r.choice([8, 24, 64, 80]),
+                               "tau": r.choice([1.0, 4.0, 16.0, 64.0]), "rank": r.choice([2, 8, 16])}}
+        layers.append({"type": kind, "mixer": mixer, "mlp": r.choice([None, {"kind": "dense", "ff": r.choice([16, 56, 104])}])})
+    return {"architecture": "Sozopel", "vocab": r.choice([50, 97, 160]), "width": width, "max_positions": 200,
+            "norm": {"eps": r.choice([1e-6, 1e-5, 1e-3])}, "canon": {"taps": r.randint(1, 6)}, "layers": layers}
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_configurations_drawn_at_random(seed, tmp_path):
+    from xeno_rt_amd.engine import Engine
+    raw = random_configuration(seed)
+    folder = make_sozopel_folder(raw, tmp_path / "model", seed=seed, keep_rank=seed % 2 == 0)
+    plain = P.PlainModel(folder)
+    ids, other = token_ids(raw["vocab"], 110, seed=seed), token_ids(raw["vocab"], 45, seed=seed + 50)
+    want, want_other = plain.logits(ids), plain.logits(other)
+    for dtype in DTYPES:
+        engine = Engine.load(folder, dtype=dtype, max_tokens=64 * 6, max_slots=2)
+        what = f"drawn {seed}: {[layer['type'] for layer in raw['layers']]}"
+        assert_logits(run_whole(engine, ids), want, dtype, what + " whole")
+        assert_logits(in_portions(engine, ids, [70, 2, 1]), want, dtype, what + " in portions and decoded")
+        got = run_batched(engine, [ids, other], [80, 3])
+        assert_logits(got[0], want, dtype, what + " batched")
+        assert_logits(got[1], want_other, dtype, what + " batched, the other")
+        engine.cache.check()
