@@ -27,9 +27,8 @@ LENGTH = {"mixed": 150, "wide": 140, "one_tap": 90}
 # cancels (the first tokens of a sequence, whose state holds one or two keys), the rounding of that sum is scaled up
 # with it, so single logits, and the root mean square over a sequence of one or two tokens, differ by more than the
 # sums' own rounding (largest seen: 2.8e-5 and 8.8e-6, on a one-token sequence).
-# In bfloat16 the same happens to the rounding of q and k themselves: single logits of the configurations drawn at random (width
-# 136, weights of deviation 0.2) are off by up to 1.3e-1 where the root mean square is 1e-2.
-LIMITS = {"float32": dict(max=1e-4, rms=2e-5), "bfloat16": dict(max=1.5e-1, rms=2.5e-2)}
+# In bfloat16 the same happens to the rounding of q and k themselves, so single logits stand out from a root mean square of 1e-2.
+LIMITS = {"float32": dict(max=1e-4, rms=2e-5), "bfloat16": dict(max=1e-1, rms=2.5e-2)}
 WORST = {}
 
 
@@ -473,10 +472,6 @@ def test_small_operations(ops):
     assert torch.equal(got.cpu(), x + table[ids.long()])
 
 
-def test_the_largest_errors_seen_are_reported():
-    print("largest errors against the plain model (max, rms):", {k: [f"{x:.2e}" for x in v] for k, v in WORST.items()})
-
-
 # ---- through the programs a user runs ----------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -550,7 +545,8 @@ def random_configuration(seed):
 def test_configurations_drawn_at_random(seed, tmp_path):
     from xeno_rt_amd.engine import Engine
     raw = random_configuration(seed)
-    folder = make_sozopel_folder(raw, tmp_path / "model", seed=seed, keep_rank=seed % 2 == 0)
+    # (matrices of deviation 0.1: with 0.2, as in the fixed configurations, the widest of these models round single logits by 16 % in bfloat16)
+    folder = make_sozopel_folder(raw, tmp_path / "model", seed=seed, std=0.1, keep_rank=seed % 2 == 0)
     plain = P.PlainModel(folder)
     ids, other = token_ids(raw["vocab"], 110, seed=seed), token_ids(raw["vocab"], 45, seed=seed + 50)
     want, want_other = plain.logits(ids), plain.logits(other)
@@ -563,3 +559,7 @@ def test_configurations_drawn_at_random(seed, tmp_path):
         assert_logits(got[0], want, dtype, what + " batched")
         assert_logits(got[1], want_other, dtype, what + " batched, the other")
         engine.cache.check()
+
+
+def test_the_largest_errors_seen_are_reported():
+    print("largest errors against the plain model (max, rms):", {k: [f"{x:.2e}" for x in v] for k, v in WORST.items()})
