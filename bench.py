@@ -109,7 +109,7 @@ def sozopel_config(size, layers, max_positions):
         "parallel": {"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
                      "mixer": {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": d, "vdim": d, "conv": 4,
                                         "mask": {"size": 512}, "scale": d ** -0.5},
-                               "right": {"heads": max(1, heads // 2), "dim": d, "vdim": 2 * d, "tau": 16.0, "rank": 16}}},
+                               "right": {"heads": max(1, heads // 2), "dim": d, "vdim": 2 * d, "tau": 8.0, "rank": 16}}},
         "retention": {"type": "retention", "mlp": None,
                       "mixer": {"heads": max(1, heads // 2), "dim": d, "vdim": 2 * d,
                                 "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(max(1, heads // 2))]}},

@@ -26,7 +26,7 @@ WIDE = {
         {"type": "parallel", "mlp": None,
          "mixer": {"left": {"heads": 2, "kv_heads": 2, "dim": 32, "vdim": 32, "conv": 4, "mask": {"size": 70}, "scale": 0.2},
                    "right": {"heads": 1, "dim": 32, "vdim": 136, "tau": 1.0, "rank": 4}}},
-        {"type": "retention", "mlp": None, "mixer": {"heads": 1, "dim": 8, "vdim": 72, "decay": [0.96875]}},
+        {"type": "retention", "mlp": None, "mixer": {"heads": 1, "dim": 8, "vdim": 72, "decay": [0.953125]}},
         {"type": "parallel", "mlp": {"kind": "dense", "ff": 40},
          "mixer": {"left": {"heads": 4, "kv_heads": 1, "dim": 16, "vdim": 8, "conv": 1, "mask": {"size": 3}, "scale": 1.0},
                    "right": {"heads": 2, "dim": 136, "vdim": 16, "tau": 30.0, "rank": 16}}},
