@@ -87,7 +87,8 @@ template <typename T, int G, int OWNED>
 __device__ __forceinline__ void attend_blocks(Seen<OWNED> (&seen)[G], int b_begin, int b_end, int first, int pos, const float* qs, float* ps,
                                               const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                               const int* __restrict__ table, int n_blocks, int n_kv_heads, int kv_head, int head_dim, int value_dim,
-                                              float scale, bool biased, const float (&slopes)[G], bool whole_pieces) {
+                                              float scale, bool biased, const float (&slopes)[G], bool whole_pieces,
+                                              const float* __restrict__ distance_bias, int bias_span, int head0) {
     const int lane = threadIdx.x % XRT_WAVE;
     for (int b = b_begin; b <= b_end; ++b) {
         const int block = table[b];
@@ -134,6 +135,7 @@ __device__ __forceinline__ void attend_blocks(Seen<OWNED> (&seen)[G], int b_begi
             for (int g = 0; g < G; ++g) {
                 s[g] = dot[g] * scale;
                 if (biased) s[g] = fmaf(slopes[g], (float)(j - pos), s[g]);
+                if (distance_bias != nullptr) s[g] += distance_bias[(long)(head0 + g) * bias_span + min(pos - j, bias_span - 1)];
             }
         }
         float correction[G];
@@ -192,7 +194,8 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
     const T* __restrict__ qkv, int row_width, int n_heads, int n_kv_heads, int head_dim, int value_dim,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_stride, int n_blocks, const int* __restrict__ positions, const int* __restrict__ slots,
-    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink, int chunk_blocks) {
+    T* __restrict__ out, float scale, int window, const float* __restrict__ distance_slopes, int sink, int chunk_blocks,
+    const float* __restrict__ distance_bias, int bias_span) {
     __shared__ float qs[G * OWNED * XRT_WAVE];                 // [G][head_dim]
     __shared__ float ps[WAVES][G * XRT_WAVE];
     // what the wavefronts found in the chunks of a round, for the merge: two sets, used in turn (WAVES > 1)
@@ -233,7 +236,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
             for (int g = 0; g < G; ++g) here[g].clear();
             attend_blocks<T, G, OWNED>(here, max(first_block, chunk * chunk_blocks), min(last_block, chunk * chunk_blocks + chunk_blocks - 1),
                                        first, pos, qs, ps[0], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, value_dim, scale,
-                                       biased, slopes, whole_pieces);
+                                       biased, slopes, whole_pieces, distance_bias, bias_span, head0);
 #pragma unroll
             for (int g = 0; g < G; ++g) merge(all[g], here[g]);
         }
@@ -250,7 +253,7 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
                 for (int g = 0; g < G; ++g) here[g].clear();
                 attend_blocks<T, G, OWNED>(here, max(first_block, chunk * chunk_blocks), min(last_block, chunk * chunk_blocks + chunk_blocks - 1),
                                            first, pos, qs, ps[wave], k_cache, v_cache, table, n_blocks, n_kv_heads, kv_head, head_dim, value_dim, scale,
-                                           biased, slopes, whole_pieces);
+                                           biased, slopes, whole_pieces, distance_bias, bias_span, head0);
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
 #pragma unroll
@@ -298,7 +301,9 @@ __global__ void __launch_bounds__(WAVES * XRT_WAVE) attention_generic_kernel(
 int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale,
-                          int window, const float* distance_slopes, int sink, hipStream_t s) {
+                          int window, const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
+                          hipStream_t s) {
+    XRT_REQUIRE(distance_bias == nullptr || bias_span > 0, "attention: a table of biases by distance needs a distance at least");
     XRT_REQUIRE(head_dim <= MAX_HEAD_DIM && value_dim > 0 && value_dim <= MAX_HEAD_DIM, "attention: head sizes %d and %d must be at most %d", head_dim, value_dim, MAX_HEAD_DIM);
     // Query heads of a key/value head that a wavefront takes together: as many of the group as 4, for head sizes up to 128
     // (what a lane then owns of a head fits two registers a head), where that still leaves two workgroups to a compute
@@ -308,7 +313,9 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
     if ((long)tokens * (n_heads / together) < 2L * XRT_COMPUTE_UNITS) together = 1;
     const long items = (long)tokens * (n_heads / together);
     XRT_REQUIRE((long)tokens * n_heads < (1L << 31), "attention: too many (token, head) pairs");
-    const int row_width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim;
+    // rows of q, k and v side by side unless the caller says how far the rows of q lie apart
+    XRT_REQUIRE(q_stride == 0 || (q_stride >= (long)n_heads * head_dim && q_stride < (1L << 31)), "attention: rows of q %ld apart", q_stride);
+    const int row_width = q_stride > 0 ? (int)q_stride : (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim;
     // few (token, head) pairs (a decode step): a workgroup of wavefronts each, which take the chunks of keys side by side
     const bool side_by_side = (long)tokens * n_heads <= 8L * XRT_COMPUTE_UNITS;
     const int chunk_blocks = window > 0 && window <= WINDOW_FOR_SHORT_CHUNKS ? 1 : CHUNK_BLOCKS;
@@ -316,7 +323,7 @@ int xrt_attention_generic(const void* qkv, int dtype, int tokens, int n_heads, i
 #define XRT_GENERIC(T, WAVES_, G_, OWNED_)                                                                                \
     attention_generic_kernel<T, WAVES_, G_, OWNED_><<<(unsigned)items, WAVES_ * XRT_WAVE, WAVES_ > 1 ? round_bytes : 0, s>>>( \
         (const T*)qkv, row_width, n_heads, n_kv_heads, head_dim, value_dim, (const T*)k_cache, (const T*)v_cache, block_table,       \
-        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink, chunk_blocks)
+        table_stride, n_blocks, positions, slots, (T*)out, scale, window, distance_slopes, sink, chunk_blocks, distance_bias, bias_span)
 #define XRT_GENERIC_WAVES(T, G_, OWNED_) do { if (side_by_side) XRT_GENERIC(T, CHUNK_WAVES, G_, OWNED_); else XRT_GENERIC(T, 1, G_, OWNED_); } while (0)
 #define XRT_GENERIC_SETS(T)                                                                                               \
     do {                                                                                                                  \

@@ -255,10 +255,56 @@ int xrt_kv_store(const void* k, long k_stride, const void* v, long v_stride, int
                  int table_stride, int n_blocks, void* stream);
 
 // The general attention kernel with values of a width of their own and, with sink, one more key of score 0 that has no value.
+// q_stride: 0 (rows of qkv are q, k and v side by side), or the distance between the rows of q where they lie alone (keys and
+// values are read from the cache only). distance_bias: null, or float32 [n_heads][bias_span]: a key d tokens behind the query
+// adds distance_bias[h][min(d, bias_span - 1)] to its scaled score (any bias that is a function of head and distance and
+// stays constant from some distance on).
 int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, int n_kv_heads, int head_dim, int value_dim,
                           const void* k_cache, const void* v_cache, const int* block_table, int table_stride, int n_blocks,
                           const int* positions, const int* slots, void* out, float scale, int window,
-                          const float* distance_slopes, int sink, void* stream);
+                          const float* distance_slopes, int sink, long q_stride, const float* distance_bias, int bias_span,
+                          void* stream);
+
+// Attention without a softmax: the weight of a visible key is sigmoid(score_h + head_bias[h]), not normalised over the keys;
+// before that the heads' scaled scores of a (query, key) pair are mixed, score_h <- sum_g head_mix[h][g] score_g
+// (head_mix float32 [n_heads][n_heads], or null); a head's summed values are multiplied by sigmoid(gate[token][h]) (float32
+// rows gate_stride apart, or null). q: rows of n_heads x head_dim, q_stride apart; out rows n_heads x value_dim; keys and
+// values come from the cache (the step's own included, which must have been written). window 0: none.
+int xrt_attention_sigmoid(const void* q, long q_stride, int dtype, long tokens, int n_heads, int n_kv_heads, int head_dim,
+                          int value_dim, const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
+                          int n_blocks, const int* positions, const int* slots, void* out, float scale, int window,
+                          const float* head_mix, const float* head_bias, const float* gate, long gate_stride, void* stream);
+
+// Between an attention's projection (float32 sums, rows [q heads | k heads | v heads | anything], proj_stride apart) and its
+// scores: biases ([heads * dim] each, or null); an RMS norm of every head of q and k with one weight [head_dim] each (or
+// null); a rotation of the first rot_dims dims of every head of q and k by the angles position * frequencies[pair]
+// (frequencies float32 [rot_dims / 2], or null; pairs of neighbours (2n, 2n + 1), or of halves (n, n + rot_dims / 2); cosines
+// and sines times magnitude); values_out (or null) takes the values as projected (float32 [tokens][n_kv_heads * value_dim]);
+// with values_in (same shape, or null) v <- (1 - lambda) v + lambda values_in, lambda one number on the device; q goes to
+// q_out (element type `dtype`, rows q_stride apart), k and v into the cache (or nowhere, if the caches are null). Biases, norm
+// weights and lambda have the element type small_dtype.
+int xrt_qkv_complete(const float* proj, long proj_stride, int dtype, long tokens, int n_heads, int n_kv_heads, int head_dim,
+                   int value_dim, const void* bias_q, const void* bias_k, const void* bias_v, const void* norm_q,
+                   const void* norm_k, float norm_eps, int small_dtype, const float* frequencies, int rot_dims,
+                   int neighbours, float magnitude, const float* values_in, float* values_out, const void* lambda,
+                   const int* positions, const int* slots, void* q_out, long q_stride, void* k_cache, void* v_cache,
+                   const int* block_table, int table_stride, int n_blocks, void* stream);
+
+// Layer norm of whole rows, y = (x - mean) / sqrt(mean of squared deviations + eps) * weight + bias; x float32, weight and
+// bias of w_dtype. xrt_layernorm: out[r] = norm(x[rows ? rows[r] : r]).
+int xrt_layernorm(const float* x, const void* weight, const void* bias, int w_dtype, float eps, void* out, int out_dtype,
+                  const int* rows, int n_rows, int hidden, void* stream);
+// The norm h of every row, then out[r] = h[r] + (h_before - h[r]) * mix, where h_before is the norm of the row before it if
+// that row is a token of the same sequence (token_slots), else the sequence's state (state [slots][hidden] float32, zeros
+// for a sequence that starts); afterwards the state holds the norm of the sequence's last row. Padding rows (slot < 0): zeros.
+int xrt_layernorm_shift(const float* x, const void* weight, const void* bias, const void* mix, int w_dtype, float eps,
+                        float* state, const int* token_slots, const int* seq_offsets, const int* seq_slots, int n_seqs,
+                        int max_count, void* out, int out_dtype, int n_rows, int hidden, void* stream);
+// residual[r] += scale * norm(y[r] + pre_bias) (pre_bias [hidden] or null); with next_out the kernel goes on to
+// next_out[r] = the layer norm (next_weight, next_bias, next_eps) of the row of the residual it has just written.
+int xrt_add_layernormed(float* residual, const float* y, const void* pre_bias, const void* weight, const void* bias, int w_dtype,
+                        float eps, float scale, const void* next_weight, const void* next_bias, float next_eps, void* next_out,
+                        int out_dtype, long rows, int hidden, void* stream);
 
 #ifdef __cplusplus
 }

@@ -69,7 +69,8 @@ class ModelSpec:
         return all(part.capturable for part in self.parts())
 
     def ignored_names(self) -> List[str]:
-        return list(self.head.ignored_names())
+        """Tensors that a checkpoint may carry and that no part reads."""
+        return [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
 
     def cache_needs(self) -> List[Optional[CacheNeeds]]:
         """For each schedule entry what its cache entry holds, None if it reads another's."""

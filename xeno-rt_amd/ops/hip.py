@@ -181,7 +181,8 @@ class HipOps:
                      "xrt_linear_with", "xrt_pack_weight", "xrt_packing_suits", "xrt_block_tokens",
                      "xrt_attention_finishes_qkv", "xrt_attention_finishing", "xrt_rope_table", "xrt_short_conv",
                      "xrt_linear_recurrence", "xrt_add_normed", "xrt_activation", "xrt_rows_add", "xrt_kv_store",
-                     "xrt_attention_general", "xrt_rmsnorm_conv_step"):
+                     "xrt_attention_general", "xrt_rmsnorm_conv_step", "xrt_attention_sigmoid", "xrt_qkv_complete",
+                     "xrt_layernorm", "xrt_layernorm_shift", "xrt_add_layernormed"):
             getattr(self.lib, name).restype = ctypes.c_int
         from ..cache.allocator import BLOCK_TOKENS
         if int(self.lib.xrt_block_tokens()) != BLOCK_TOKENS:
@@ -464,16 +465,19 @@ class HipOps:
                                                         0 if rope_table is None else int(rope_table.shape[0]), int(batch.max_context)))
 
     def attention(self, qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, window=None, distance_slopes=None,
-                  finish: Optional[QkvFinish] = None, value_dim: Optional[int] = None, sink: bool = False):
+                  finish: Optional[QkvFinish] = None, value_dim: Optional[int] = None, sink: bool = False,
+                  distance_bias: Optional[torch.Tensor] = None, queries_alone: bool = False):
         """Causal attention of the step's tokens over the cache. distance_slopes: float32 [n_heads], or None; a key at
-        position j adds slope * (j - P) to the scaled score of the query at position P. finish: what is still to do to
+        position j adds slope * (j - P) to the scaled score of the query at position P. distance_bias: float32
+        [n_heads, span], or None; a key d tokens behind the query adds distance_bias[h, min(d, span - 1)]. queries_alone: the
+        rows of `qkv` hold the queries only (keys and values are in the cache already). finish: what is still to do to
         q, k and v (only where `attention_finishes_qkv` says so); the cache must be writable then."""
         from ..cache import BLOCK_TOKENS
         if finish is not None:
             return self._attention_finishing(qkv, n_heads, n_kv_heads, head_dim, kv, batch, out, scale, finish)
-        if sink or (value_dim is not None and value_dim != head_dim):
+        if sink or (value_dim is not None and value_dim != head_dim) or distance_bias is not None or queries_alone:
             return self._attention_general(qkv, n_heads, n_kv_heads, head_dim, value_dim or head_dim, kv, batch, out, scale, window,
-                                           distance_slopes, sink)
+                                           distance_slopes, sink, distance_bias, queries_alone)
         tokens = qkv.shape[0]
         width = (n_heads + 2 * n_kv_heads) * head_dim
         self._require(qkv, "qkv", None, (tokens, width))
@@ -507,11 +511,20 @@ class HipOps:
             ctypes.c_float(scale), int(window or 0), _ptr(distance_slopes), _ptr(offsets), _ptr(seq_slots), _ptr(starts), n_seqs,
             max_count, max_context, _ptr(workspace), ctypes.c_long(workspace_floats), self._stream(qkv)))
 
-    def _attention_general(self, qkv, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window, distance_slopes, sink):
-        """Rows of qkv are [n_heads x head_dim | n_kv_heads x head_dim | n_kv_heads x value_dim], rows of out n_heads x value_dim.
-        sink: the softmax's denominator has one more (a key of score 0 without a value)."""
+    def _attention_general(self, qkv, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window, distance_slopes, sink,
+                           distance_bias=None, queries_alone=False):
+        """Rows of qkv are [n_heads x head_dim | n_kv_heads x head_dim | n_kv_heads x value_dim] (or the queries alone), rows of
+        out n_heads x value_dim. sink: the softmax's denominator has one more (a key of score 0 without a value)."""
         tokens = qkv.shape[0]
-        self._require(qkv, "qkv", None, (tokens, (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim))
+        q_stride = 0
+        if queries_alone:
+            q_stride = self._rows(qkv, "attention q", n_heads * head_dim)
+        else:
+            self._require(qkv, "qkv", None, (tokens, (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim))
+        span = 0
+        if distance_bias is not None:
+            span = distance_bias.shape[-1]
+            self._require(distance_bias, "attention distance_bias", torch.float32, (n_heads, span), qkv)
         self._require(out, "attention out", qkv.dtype, (tokens, n_heads * value_dim), qkv)
         self._require(batch.positions, "positions", torch.int32, (tokens,), qkv)
         self._require(batch.slots, "slots", torch.int32, (tokens,), qkv)
@@ -521,7 +534,136 @@ class HipOps:
         self._check(self.lib.xrt_attention_general(
             _ptr(qkv), _code(qkv), tokens, n_heads, n_kv_heads, head_dim, value_dim, _ptr(k_cache), _ptr(v_cache), _ptr(table), stride,
             n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale), int(window or 0),
-            _ptr(distance_slopes), int(bool(sink)), self._stream(qkv)))
+            _ptr(distance_slopes), int(bool(sink)), ctypes.c_long(q_stride), _ptr(distance_bias), int(span), self._stream(qkv)))
+
+    def attention_sigmoid(self, q, n_heads, n_kv_heads, head_dim, value_dim, kv, batch, out, scale, window=None, head_mix=None,
+                          head_bias=None, gate=None):
+        """Attention whose weights are sigmoid(score + head_bias[h]) of every visible key, not normalised over the keys. q: rows
+        of n_heads x head_dim (they may be columns of a wider matrix); the keys and values of the step are in the cache already.
+        head_mix: float32 [n_heads, n_heads], the heads' scaled scores of a (query, key) pair are multiplied by it before the
+        sigmoid; head_bias: float32 [n_heads]; gate: float32 rows with one number per head (columns of a wider matrix, if
+        need be): a head's output is multiplied by sigmoid(gate)."""
+        tokens = q.shape[0]
+        q_stride = self._rows(q, "attention q", n_heads * head_dim)
+        self._require(out, "attention out", q.dtype, (tokens, n_heads * value_dim), q)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), q)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), q)
+        k_cache, v_cache, table, stride, n_blocks = self._kv(kv, q, n_kv_heads, head_dim, value_dim)
+        if head_mix is not None:
+            self._require(head_mix, "attention head_mix", torch.float32, (n_heads, n_heads), q)
+        if head_bias is not None:
+            self._require(head_bias, "attention head_bias", torch.float32, (n_heads,), q)
+        gate_stride = 0 if gate is None else self._rows(gate, "attention gate", n_heads, torch.float32, q)
+        self._check(self.lib.xrt_attention_sigmoid(
+            _ptr(q), ctypes.c_long(q_stride), _code(q), ctypes.c_long(tokens), n_heads, n_kv_heads, head_dim, value_dim, _ptr(k_cache),
+            _ptr(v_cache), _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale),
+            int(window or 0), _ptr(head_mix), _ptr(head_bias), _ptr(gate), ctypes.c_long(gate_stride), self._stream(q)))
+
+    def qkv_complete(self, proj, n_heads, n_kv_heads, head_dim, value_dim, batch, q_out, kv=None, biases=None, norms=None,
+                     norm_eps=0.0, frequencies=None, rot_dims=0, neighbours=True, magnitude=1.0, values_in=None, values_out=None,
+                     blend=None):
+        """What lies between an attention's projection and its scores. proj: float32 rows [q | k | v | ...] (the leading columns
+        of the projection's output). biases: (q, k, v) vectors or None; norms: (q, k) weights [head_dim] of an RMS norm of every
+        head, or None; frequencies: float32 [rot_dims / 2], the first rot_dims dims of every head of q and k turn by
+        position * frequency in pairs of neighbours (or of halves), cosines and sines times magnitude; values_out: float32
+        [tokens, n_kv_heads * value_dim] takes the values as projected; values_in (same shape) with blend (one number on the
+        device): v <- (1 - blend) v + blend values_in. q goes to q_out (compute dtype), k and v into the cache `kv` (if given)."""
+        tokens = proj.shape[0]
+        width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
+        if proj.dim() != 2 or proj.shape[1] < width:
+            raise KernelError(f"qkv_complete proj: {tuple(proj.shape)}, expected at least {width} columns")
+        proj_stride = self._rows(proj, "qkv_complete proj", None, torch.float32)
+        q_stride = self._rows(q_out, "qkv_complete q_out", n_heads * head_dim, None, proj)
+        self._require(batch.positions, "positions", torch.int32, (tokens,), proj)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), proj)
+        small = [t for t in (*(biases or ()), *(norms or ()), blend) if t is not None]
+        small_dtype = small[0].dtype if small else torch.float32
+        b_q = b_k = b_v = n_q = n_k = None
+        if biases is not None:
+            b_q, b_k, b_v = biases
+            self._require(b_q, "qkv_complete bias of q", small_dtype, (n_heads * head_dim,), proj)
+            self._require(b_k, "qkv_complete bias of k", small_dtype, (n_kv_heads * head_dim,), proj)
+            self._require(b_v, "qkv_complete bias of v", small_dtype, (n_kv_heads * value_dim,), proj)
+        if norms is not None:
+            n_q, n_k = norms
+            self._require(n_q, "qkv_complete norm of q", small_dtype, (head_dim,), proj)
+            self._require(n_k, "qkv_complete norm of k", small_dtype, (head_dim,), proj)
+        if frequencies is not None:
+            self._require(frequencies, "qkv_complete frequencies", torch.float32, (rot_dims // 2,), proj)
+        for what, tensor in (("values_in", values_in), ("values_out", values_out)):
+            if tensor is not None:
+                self._require(tensor, f"qkv_complete {what}", torch.float32, (tokens, n_kv_heads * value_dim), proj)
+        if values_in is not None:
+            if blend is None or blend.numel() != 1:
+                raise KernelError("qkv_complete: values to blend in need their share, one number on the device")
+            self._require(blend, "qkv_complete blend", small_dtype, None, proj)
+        k_cache = v_cache = table = None
+        stride = n_blocks = 0
+        if kv is not None:
+            k_cache, v_cache, table, stride, n_blocks = self._kv(kv, q_out, n_kv_heads, head_dim, value_dim)
+        self._check(self.lib.xrt_qkv_complete(
+            _ptr(proj), ctypes.c_long(proj_stride), _code(q_out), ctypes.c_long(tokens), n_heads, n_kv_heads, head_dim, value_dim,
+            _ptr(b_q), _ptr(b_k), _ptr(b_v), _ptr(n_q), _ptr(n_k), ctypes.c_float(norm_eps), _CODES[small_dtype], _ptr(frequencies),
+            int(rot_dims), int(bool(neighbours)), ctypes.c_float(magnitude), _ptr(values_in), _ptr(values_out), _ptr(blend),
+            _ptr(batch.positions), _ptr(batch.slots), _ptr(q_out), ctypes.c_long(q_stride), _ptr(k_cache), _ptr(v_cache), _ptr(table),
+            stride, n_blocks, self._stream(proj)))
+
+    # -- layer norm ---------------------------------------------------------------------------------
+    def layernorm(self, x, weight, bias, eps, out, rows=None):
+        """out = (x - mean) / sqrt(var + eps) * weight + bias over whole rows (only `rows` of x, if given); x float32."""
+        hidden = x.shape[-1]
+        self._require(x, "layernorm x", torch.float32)
+        if x.dim() != 2:
+            raise KernelError("layernorm x: expected [rows, hidden]")
+        n_rows = x.shape[0] if rows is None else rows.shape[0]
+        self._require(weight, "layernorm weight", None, (hidden,), x)
+        self._require(bias, "layernorm bias", weight.dtype, (hidden,), x)
+        self._require(out, "layernorm out", None, (n_rows, hidden), x)
+        if rows is not None:
+            self._require(rows, "layernorm rows", torch.int32, (n_rows,), x)
+        self._check(self.lib.xrt_layernorm(_ptr(x), _ptr(weight), _ptr(bias), _code(weight), ctypes.c_float(eps), _ptr(out), _code(out),
+                                           _ptr(rows), n_rows, hidden, self._stream(x)))
+
+    def layernorm_shift(self, x, weight, bias, eps, mix, state, batch, out):
+        """The layer norm h of every row, then out = h + (h of the token before - h) * mix along each sequence; state
+        [slots, hidden] float32 holds the last h of every sequence (zeros when it starts) and is brought up to date."""
+        tokens, hidden = x.shape
+        self._require(x, "layernorm_shift x", torch.float32)
+        self._require(weight, "layernorm_shift weight", None, (hidden,), x)
+        self._require(bias, "layernorm_shift bias", weight.dtype, (hidden,), x)
+        self._require(mix, "layernorm_shift mix", weight.dtype, (hidden,), x)
+        self._require(state, "layernorm_shift state", torch.float32, (state.shape[0], hidden), x)
+        self._require(out, "layernorm_shift out", None, (tokens, hidden), x)
+        self._require(batch.slots, "slots", torch.int32, (tokens,), x)
+        offsets, slots, n = self._sequences(batch, tokens, x)
+        self._check(self.lib.xrt_layernorm_shift(_ptr(x), _ptr(weight), _ptr(bias), _ptr(mix), _code(weight), ctypes.c_float(eps),
+                                                 _ptr(state), _ptr(batch.slots), offsets, slots, n, int(batch.max_count), _ptr(out),
+                                                 _code(out), tokens, hidden, self._stream(x)))
+
+    def add_layernormed(self, residual, y, weight, bias, eps, scale=1.0, pre_bias=None, then=None, then_out=None):
+        """residual += scale * layer_norm(y + pre_bias); y float32 like residual. then = (weight, bias, eps) of a layer norm of
+        the updated residual, written to then_out in the same pass."""
+        self._require(residual, "add_layernormed residual", torch.float32)
+        if residual.dim() != 2:
+            raise KernelError("add_layernormed: a residual [rows, width]")
+        rows, width = residual.shape
+        self._require(y, "add_layernormed y", torch.float32, (rows, width), residual)
+        self._require(weight, "add_layernormed weight", None, (width,), residual)
+        self._require(bias, "add_layernormed bias", weight.dtype, (width,), residual)
+        if pre_bias is not None:
+            self._require(pre_bias, "add_layernormed pre_bias", weight.dtype, (width,), residual)
+        next_w = next_b = None
+        next_eps, out_code = 0.0, 0
+        if then is not None:
+            next_w, next_b, next_eps = then
+            self._require(next_w, "add_layernormed next weight", weight.dtype, (width,), residual)
+            self._require(next_b, "add_layernormed next bias", weight.dtype, (width,), residual)
+            self._require(then_out, "add_layernormed then_out", None, (rows, width), residual)
+            out_code = _code(then_out)
+        self._check(self.lib.xrt_add_layernormed(_ptr(residual), _ptr(y), _ptr(pre_bias), _ptr(weight), _ptr(bias), _code(weight),
+                                                 ctypes.c_float(eps), ctypes.c_float(scale), _ptr(next_w), _ptr(next_b),
+                                                 ctypes.c_float(next_eps), _ptr(then_out if then is not None else None), out_code,
+                                                 ctypes.c_long(rows), width, self._stream(residual)))
 
     # -- mixing along the sequence with state of fixed size ----------------------------
     def _rows(self, tensor, what, width=None, dtype=None, like=None):

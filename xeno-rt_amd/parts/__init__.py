@@ -1,14 +1,14 @@
 """Parts that models are built from."""
 from .base import (Block, CacheNeeds, FeedForward, HalfSplitRotation, KVSpec, Mixer, Norm, Part, PositionEncoding,
                    Runtime, StateSpec, WeightSpec, create_part, register_part, registered_parts)
-from .norm import RMSNorm, ScalarRMSNorm
-from .position import DistanceSlopes, NoPosition, Rotary
+from .norm import LayerNorm, RMSNorm, ScalarRMSNorm
+from .position import DistanceBuckets, DistanceSlopes, NoPosition, PairRotation, Rotary
 from .convolution import ShortConvolution, TokenShift
-from .attention import Attention
+from .attention import Attention, SharedValues
 from .recurrent import GatedLinearAttention, Retention, TimeMixWKV
 from .parallel import ParallelMixer
 from .feedforward import DenseMLP, GatedMLP
-from .block import PreNormBlock
+from .block import PreNormBlock, SandwichBlock
 from .embedding import Embedding, OutputHead, PositionedEmbedding
 
 __all__ = [
@@ -16,5 +16,6 @@ __all__ = [
     "Runtime", "StateSpec", "WeightSpec", "create_part", "register_part", "registered_parts",
     "RMSNorm", "NoPosition", "Rotary", "Attention", "GatedMLP", "PreNormBlock", "Embedding", "OutputHead",
     "ScalarRMSNorm", "DistanceSlopes", "ShortConvolution", "TokenShift", "GatedLinearAttention", "Retention", "TimeMixWKV",
-    "ParallelMixer", "DenseMLP", "PositionedEmbedding",
+    "ParallelMixer", "DenseMLP", "PositionedEmbedding", "LayerNorm", "DistanceBuckets", "PairRotation", "SharedValues",
+    "SandwichBlock",
 ]

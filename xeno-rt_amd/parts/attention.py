@@ -18,6 +18,17 @@ sequence), a softmax with one more in its denominator (`sink`: a key of score 0 
 position encoding that biases the scores by distance, and tensor names of the caller's choice (`names`). With any of
 the first three the step takes the general attention kernel, and the keys and values reach the cache through a
 kernel of their own.
+
+Further options make the step take the completed path (`_attend_completed`): one projection for q, k, v (and the
+output gate) with float32 sums, one kernel that completes them (biases, head norms, a rotation of pairs by a table of
+frequencies, the blend of the values with another layer's, the cache write), then the attention kernel that the
+weights ask for. These options are: biases on the four projections (`biases`); weights that are sigmoid(score) of
+every visible key instead of a softmax over them (`weights="sigmoid"`), with the heads' scores of a pair mixed by a
+matrix (`head_mix`) and a number per head added (`score_bias`) before the sigmoid; a gate per token and head on the
+heads' outputs, sigmoid of a projection of the mixer's input (`output_gate`); values blended with those that another
+attention layer made of the same token, v <- (1 - lambda) v + lambda v_other (`values=SharedValues.source()` in the
+layer whose values are kept for the step, `.reader(name)` in those that blend them in, lambda the tensor `name`); a
+position encoding that says `pair_rotation()`, or one that says `score_bias_table()`.
 """
 from __future__ import annotations
 
@@ -27,6 +38,21 @@ from typing import Dict, Optional
 import torch
 
 from .base import CacheNeeds, KVSpec, Mixer, PositionEncoding, Runtime, WeightSpec, register_part
+
+
+class SharedValues:
+    """The values that one attention layer made of a step's tokens (float32 [tokens, kv_heads * value_dim], as projected,
+    with their bias), kept while the step runs so that later layers can blend them into their own. A model makes one and
+    hands `source()` to the layer that fills it and `reader(name)` to those that read it."""
+
+    def __init__(self):
+        self.tensor = None
+
+    def source(self, unused_name: Optional[str] = None):
+        return (self, "source", unused_name)
+
+    def reader(self, blend_name: str):
+        return (self, "reader", blend_name)
 
 
 class Attention(Mixer):
@@ -41,19 +67,37 @@ class Attention(Mixer):
                  position: Optional[PositionEncoding] = None, qk_norm: bool = False,
                  qk_norm_eps: float = 0.0, scale: Optional[float] = None,
                  window: Optional[int] = None, value_dim: Optional[int] = None, sink: bool = False,
-                 convolution=None, names: Optional[Dict[str, str]] = None):
+                 convolution=None, names: Optional[Dict[str, str]] = None, biases: bool = False, weights: str = "softmax",
+                 head_mix: Optional[str] = None, score_bias: Optional[str] = None, output_gate: Optional[str] = None,
+                 values=None, unread=()):
         if n_heads <= 0 or n_kv_heads <= 0 or n_heads % n_kv_heads != 0:
             raise ValueError(f"head counts {n_heads}/{n_kv_heads}: the first must be a multiple of the second")
+        if weights not in ("softmax", "sigmoid"):
+            raise ValueError(f"the weights of the keys are 'softmax' or 'sigmoid', found {weights!r}")
+        if weights == "softmax" and (head_mix is not None or score_bias is not None):
+            raise ValueError("a mix of the heads' scores and a number per head belong to sigmoid weights")
         self.value_dim = head_dim if value_dim is None else int(value_dim)
         self.sink = bool(sink)
         self.convolution = convolution
-        self.general = self.sink or self.value_dim != head_dim or convolution is not None
+        self.biases, self.weights = bool(biases), weights
+        self.head_mix_name, self.score_bias_name, self.gate_name = head_mix, score_bias, output_gate
+        self.values = values
+        self.unread = tuple(unread)         # tensors under the prefix that a checkpoint may carry and this layer does not read
+        self.completed = (self.biases or weights == "sigmoid" or output_gate is not None or values is not None
+                          or hasattr(position, "pair_rotation") or hasattr(position, "score_bias_table"))
+        if self.completed and (self.sink or convolution is not None):
+            raise ValueError("the completed path of attention has neither sink nor convolution")
+        if weights == "sigmoid" and hasattr(position, "score_bias_table"):
+            raise ValueError("a bias by distance is served for softmax weights")
+        self.general = self.completed or self.sink or self.value_dim != head_dim or convolution is not None
         if head_dim <= 0 or (head_dim % 2 != 0 and not self.general):   # llama.rs:125-128 takes any size; the rotation pairs dims, so an even one
             raise ValueError(f"head_dim {head_dim} must be positive and even")
-        if self.general and qk_norm:
+        if self.general and qk_norm and not self.completed:
             raise ValueError("attention with a sink, a convolution or values of another width takes no head norms")
         self.names = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                       "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", **(names or {})}
+        for name in "qkvo":                                             # a projection's bias, unless the caller names it
+            self.names.setdefault(name + "_bias", self.names[name].replace(".weight", "") + ".bias")
         self.prefix = prefix
         self.hidden = hidden
         self.n_heads = n_heads
@@ -85,7 +129,29 @@ class Attention(Mixer):
             specs[p + n["k_norm"]] = WeightSpec((self.head_dim,), init="ones", kind="vector")
         if self.convolution is not None:
             specs.update(self.convolution.weight_specs())
+        if self.biases:
+            for name, width in (("q", self.q_width), ("k", self.kv_width), ("v", self.v_width), ("o", self.hidden)):
+                specs[p + n[name + "_bias"]] = WeightSpec((width,), init="zeros", kind="vector")
+        if self.head_mix_name is not None:
+            specs[p + self.head_mix_name] = WeightSpec((self.n_heads, self.n_heads), kind="vector")
+        if self.score_bias_name is not None:
+            specs[p + self.score_bias_name] = WeightSpec((self.n_heads,), init="zeros", kind="vector")
+        if self.gate_name is not None:
+            specs[p + self.gate_name] = WeightSpec((self.n_heads, self.hidden))
+        if self.values is not None and self.values[2] is not None:
+            specs[p + self.values[2]] = WeightSpec((), init="zeros", kind="vector")
+        if self.completed and self.position is not None:
+            specs.update(self.position.weight_specs())
         return specs
+
+    @property
+    def has_output_bias(self) -> bool:
+        return self.biases
+
+    def ignored_names(self):
+        """Tensors that a checkpoint may carry for this layer and that it does not read (the share of a blend in a layer
+        that blends nothing in, for one)."""
+        return [self.prefix + name for name in self.unread]
 
     def cache_needs(self) -> CacheNeeds:
         needs = CacheNeeds(kv=KVSpec(self.n_kv_heads, self.head_dim, self.window,
@@ -97,6 +163,23 @@ class Attention(Mixer):
         p, n = self.prefix, self.names
         if self.position is not None:
             self.position.bind(tensors, runtime)
+        if self.completed:
+            self.w_proj = runtime.weight([tensors[p + n[name]] for name in "qkv"]
+                                         + ([tensors[p + self.gate_name]] if self.gate_name is not None else []))
+            self.w_o = runtime.weight(tensors[p + n["o"]])
+            self.bias_qkv = self.bias_o = self.head_norms = self.head_mix = self.score_bias = self.blend = None
+            if self.biases:
+                self.bias_qkv = tuple(runtime.vector(tensors[p + n[name + "_bias"]]) for name in "qkv")
+                self.bias_o = runtime.vector(tensors[p + n["o_bias"]])
+            if self.qk_norm:
+                self.head_norms = (runtime.vector(tensors[p + n["q_norm"]]), runtime.vector(tensors[p + n["k_norm"]]))
+            if self.head_mix_name is not None:
+                self.head_mix = tensors[p + self.head_mix_name].to(device=runtime.device, dtype=torch.float32).contiguous()
+            if self.score_bias_name is not None:
+                self.score_bias = tensors[p + self.score_bias_name].to(device=runtime.device, dtype=torch.float32).contiguous()
+            if self.values is not None and self.values[1] == "reader":
+                self.blend = runtime.vector(tensors[p + self.values[2]]).reshape(1)
+            return
         if self.general:
             if self.position is not None and self.position.rotation() is not None:
                 raise ValueError("attention with a sink, a convolution or values of another width takes no rotation")
@@ -135,14 +218,67 @@ class Attention(Mixer):
                       distance_slopes=slopes, value_dim=self.value_dim, sink=self.sink)
         return out
 
-    def forward_into(self, h, batch, cache, out: torch.Tensor) -> None:
+    def _attend_completed(self, h, batch, cache):
+        """The heads' outputs [tokens, n_heads * value_dim] on the completed path."""
+        rt = self.runtime
+        ops = rt.ops
+        tokens = h.shape[0]
+        qkv_width = self.q_width + self.kv_width + self.v_width
+        proj = rt.empty((tokens, qkv_width + (self.n_heads if self.gate_name is not None else 0)), torch.float32)
+        ops.linear(h, self.w_proj, proj)
+        rotation = self.position.pair_rotation() if hasattr(self.position, "pair_rotation") else (None, 0, True, 1.0)
+        values_in = values_out = None
+        if self.values is not None:
+            link, role, _ = self.values
+            if role == "source":
+                values_out = link.tensor = rt.empty((tokens, self.v_width), torch.float32)
+            else:
+                values_in = link.tensor
+                if values_in is None or tuple(values_in.shape) != (tokens, self.v_width):
+                    raise ValueError("the values to blend in are those of an earlier layer of this step, of the same width")
+        q = rt.empty((tokens, self.q_width))
+        ops.qkv_complete(proj, self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, batch, q,
+                         kv=cache.kv if cache.writable else None, biases=self.bias_qkv, norms=self.head_norms,
+                         norm_eps=self.qk_norm_eps, frequencies=rotation[0], rot_dims=rotation[1], neighbours=rotation[2],
+                         magnitude=rotation[3], values_in=values_in, values_out=values_out, blend=self.blend)
+        out = rt.empty((tokens, self.n_heads * self.value_dim))
+        if self.weights == "sigmoid":
+            ops.attention_sigmoid(q, self.n_heads, self.n_kv_heads, self.head_dim, self.value_dim, cache.kv, batch, out, self.scale,
+                                  window=self.window, head_mix=self.head_mix, head_bias=self.score_bias,
+                                  gate=proj[:, qkv_width:] if self.gate_name is not None else None)
+            return out
+        if self.gate_name is not None:
+            raise NotImplementedError("an output gate is served with sigmoid weights")
+        table = self.position.score_bias_table() if hasattr(self.position, "score_bias_table") else None
+        slopes = None if self.position is None else self.position.score_slopes()
+        ops.attention(q, self.n_heads, self.n_kv_heads, self.head_dim, cache.kv, batch, out, scale=self.scale, window=self.window,
+                      distance_slopes=slopes, value_dim=self.value_dim, distance_bias=table, queries_alone=True)
+        return out
+
+    def forward_into(self, h, batch, cache, out: torch.Tensor, bias_later: bool = False):
         """The mixer's output into `out` (float32 [tokens, hidden]) instead of onto the residual stream: for an attention
-        that is one of several mixers side by side."""
+        that is one of several mixers side by side, or whose block puts a norm behind it. bias_later: the output
+        projection's bias is not added but returned, for a caller that adds it on its own way."""
         if not self.general:
             raise NotImplementedError("only the general path writes its output aside")
-        self.runtime.ops.linear(self._attend_general(h, batch, cache), self.w_o, out)
+        rt = self.runtime
+        if not self.completed:
+            rt.ops.linear(self._attend_general(h, batch, cache), self.w_o, out)
+            return None
+        rt.ops.linear(self._attend_completed(h, batch, cache), self.w_o, out)
+        if self.bias_o is None or bias_later:
+            return self.bias_o
+        row = rt.empty((out.shape[0],), torch.int32)
+        row.zero_()
+        rt.ops.rows_add(self.bias_o.reshape(1, -1), row, out)
+        return None
 
     def forward(self, h, batch, cache, residual: torch.Tensor, then=None):
+        if self.completed:
+            out = self.runtime.empty(residual.shape, torch.float32)
+            self.forward_into(h, batch, cache, out)
+            self.runtime.ops.add(residual, out)
+            return None
         if self.general:
             self.runtime.ops.linear(self._attend_general(h, batch, cache), self.w_o, residual, accumulate=True)
             return None

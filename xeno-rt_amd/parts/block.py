@@ -12,6 +12,8 @@ from __future__ import annotations
 
 from typing import Dict
 
+import torch
+
 from .base import Block, CacheNeeds, Runtime, WeightSpec, register_part
 
 
@@ -88,4 +90,70 @@ class PreNormBlock(Block):
         return None
 
 
+class SandwichBlock(Block):
+    """A norm before and a norm after each sublayer, and a number m that multiplies what a sublayer adds:
+    x += m * post1(mixer(read1(pre1(x)))), then, if the block has a feed-forward, x += m * post2(feed_forward(pre2(x))).
+    `mixer_input` is an input transform as in PreNormBlock. Mixer and feed-forward write their float32 output aside
+    (`forward_into`), the post norm takes it from there onto the stream (`Norm.add_to`); a mixer that has an output bias
+    and can leave it to the caller (`forward_into(..., bias_later=True)` returns it) has it added on the norm's way in,
+    and where both are layer norms the first post norm goes on to the feed-forward's norm in the same pass."""
+
+    def __init__(self, mixer_norm, mixer, mixer_post_norm, feed_forward_norm=None, feed_forward=None, feed_forward_post_norm=None,
+                 residual_scale: float = 1.0, mixer_input=None):
+        if len({feed_forward is None, feed_forward_norm is None, feed_forward_post_norm is None}) != 1:
+            raise ValueError("a feed-forward and its two norms come together")
+        self.mixer_norm, self.mixer, self.mixer_post_norm = mixer_norm, mixer, mixer_post_norm
+        self.feed_forward_norm, self.feed_forward, self.feed_forward_post_norm = feed_forward_norm, feed_forward, feed_forward_post_norm
+        self.residual_scale = float(residual_scale)
+        self.mixer_input = mixer_input
+
+    def parts(self):
+        return tuple(part for part in (self.mixer_norm, self.mixer_input, self.mixer, self.mixer_post_norm, self.feed_forward_norm,
+                                       self.feed_forward, self.feed_forward_post_norm) if part is not None)
+
+    @property
+    def capturable(self) -> bool:
+        return all(part.capturable for part in self.parts())
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        specs: Dict[str, WeightSpec] = {}
+        for part in self.parts():
+            specs.update(part.weight_specs())
+        return specs
+
+    def ignored_names(self):
+        return [name for part in self.parts() for name in getattr(part, "ignored_names", lambda: [])()]
+
+    def cache_needs(self) -> CacheNeeds:
+        return self.mixer.cache_needs().merged(*([self.mixer_input.cache_needs()] if self.mixer_input is not None else []))
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        for part in self.parts():
+            part.bind(tensors, runtime)
+
+    def first_norm(self):
+        return self.mixer_norm
+
+    def forward(self, x, batch, cache) -> None:
+        rt = self.runtime
+        h = PreNormBlock._read(x, self.mixer_norm, self.mixer_input, batch, cache)
+        y = rt.empty(x.shape, torch.float32)
+        post = self.mixer_post_norm
+        takes_bias = hasattr(post, "centred")
+        bias = self.mixer.forward_into(h, batch, cache, y, **({"bias_later": True} if takes_bias and getattr(self.mixer, "has_output_bias", False) else {}))
+        extra = {} if bias is None else {"pre_bias": bias}
+        if self.feed_forward is None:
+            post.add_to(x, y, self.residual_scale, **extra)
+            return
+        if takes_bias and hasattr(self.feed_forward_norm, "centred"):
+            h = post.add_to(x, y, self.residual_scale, then=self.feed_forward_norm, **extra)
+        else:
+            post.add_to(x, y, self.residual_scale, **extra)
+            h = self.feed_forward_norm.forward(x)
+        self.feed_forward.forward_into(h, batch, y)
+        self.feed_forward_post_norm.add_to(x, y, self.residual_scale)
+
+
 register_part("block", "pre_norm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

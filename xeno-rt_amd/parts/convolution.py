@@ -61,11 +61,15 @@ class ShortConvolution(Part):
 
 class TokenShift(Part):
     """For each of several readers its own mix of a token and the one before it: u + (u[t - 1] - u) * mu, with
-    mu [channels] per reader and zeros before the sequence's start. Returns [readers, tokens, channels]."""
+    mu [channels] per reader and zeros before the sequence's start. Returns [readers, tokens, channels], or with
+    `single` (one reader) [tokens, channels]: so it can stand as a sublayer's input transform."""
     capturable = True
 
-    def __init__(self, names: Sequence[str], channels: int, state_name: str):
+    def __init__(self, names: Sequence[str], channels: int, state_name: str, single: bool = False):
         self.names, self.channels, self.state_name = list(names), int(channels), state_name
+        if single and len(self.names) != 1:
+            raise ValueError("a token shift that returns a matrix has one reader")
+        self.single = bool(single)
         self.weight = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
@@ -81,4 +85,19 @@ class TokenShift(Part):
     def forward(self, u: torch.Tensor, batch, cache) -> torch.Tensor:
         out = self.runtime.empty((len(self.names), u.shape[0], self.channels), u.dtype)
         self.runtime.ops.short_conv(u, self.weight, cache.states[self.state_name], batch, out, mode="towards_last")
+        return out[0] if self.single else out
+
+    def forward_normed(self, x: torch.Tensor, norm, batch, cache) -> torch.Tensor:
+        """The shift of norm(x). Where there is one reader and the norm is a layer norm over whole rows, one kernel does
+        both and keeps everything float32 up to the one rounding of its result (the state then holds the normed row
+        itself, not what the compute dtype made of it; an engine takes this path in every step or in none)."""
+        rt = self.runtime
+        fused = getattr(rt.ops, "layernorm_shift", None)
+        centred = getattr(norm, "centred", None)
+        if fused is None or centred is None or not self.single or x.shape[1] != self.channels:
+            return self.forward(norm.forward(x), batch, cache)
+        weight, bias, eps = centred()
+        out = rt.empty((x.shape[0], self.channels))
+        state = cache.states[self.state_name]
+        fused(x, weight, bias, eps, self.weight[0], state.view(state.shape[0], self.channels), batch, out)
         return out

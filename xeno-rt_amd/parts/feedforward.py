@@ -21,30 +21,38 @@ class GatedMLP(FeedForward):
 
     ACTIVATIONS = ("silu",)
 
-    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu"):
+    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu",
+                 gate: str = "gate_proj.weight", up: str = "up_proj.weight", down: str = "down_proj.weight"):
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"activation must be one of {self.ACTIVATIONS}, found {activation!r}")
         self.prefix = prefix
         self.hidden = hidden
         self.intermediate = intermediate
         self.activation = activation
+        self.gate_name, self.up_name, self.down_name = prefix + gate, prefix + up, prefix + down
         self.w_gate_up = None
         self.w_down = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        p, h, i = self.prefix, self.hidden, self.intermediate
+        h, i = self.hidden, self.intermediate
         return {
-            p + "gate_proj.weight": WeightSpec((i, h)),
-            p + "up_proj.weight": WeightSpec((i, h)),
-            p + "down_proj.weight": WeightSpec((h, i)),
+            self.gate_name: WeightSpec((i, h)),
+            self.up_name: WeightSpec((i, h)),
+            self.down_name: WeightSpec((h, i)),
         }
 
     def bind(self, tensors, runtime: Runtime) -> None:
         super().bind(tensors, runtime)
-        p = self.prefix
-        self.w_gate_up = runtime.weight([tensors[p + name] for name in ("gate_proj.weight", "up_proj.weight")],
-                                        "gated", gated_n=self.intermediate)
-        self.w_down = runtime.weight(tensors[p + "down_proj.weight"])
+        self.w_gate_up = runtime.weight([tensors[self.gate_name], tensors[self.up_name]], "gated", gated_n=self.intermediate)
+        self.w_down = runtime.weight(tensors[self.down_name])
+
+    def forward_into(self, h, batch, out: torch.Tensor) -> None:
+        """The feed-forward's output into `out` (float32 [tokens, hidden]) instead of onto the residual stream: for a
+        block that puts a norm between the two."""
+        rt = self.runtime
+        act = rt.empty((h.shape[0], self.intermediate))
+        rt.ops.linear_glu(h, self.w_gate_up, act, activation=self.activation)
+        rt.ops.linear(act, self.w_down, out)
 
     def forward(self, h, batch, residual: torch.Tensor, then=None):
         rt = self.runtime

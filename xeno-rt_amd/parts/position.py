@@ -7,6 +7,9 @@ reference's crates/xrt-kernels/src/cpu/rope.rs:10-16 (table), :59-68 (angle),
 """
 from __future__ import annotations
 
+import math
+from typing import Optional
+
 import torch
 
 from .base import HalfSplitRotation, PositionEncoding, Runtime, register_part
@@ -78,6 +81,102 @@ class DistanceSlopes(PositionEncoding):
         return self.slopes
 
 
+class PairRotation(PositionEncoding):
+    """Pairs of dims of every head of q and k turn by the angle position * f_n, the first rope_dim dims of a head in
+    pairs of neighbours (2n, 2n + 1) or of halves (n, n + rope_dim / 2); the rest pass. f_n = base^(-2n / rope_dim), or
+    with `scaling` = {factor, original, fast, slow} stretched for contexts beyond the `original` length: with
+    c(t) = rope_dim ln(original / (2 pi t)) / (2 ln base) the pair at which a wave makes t turns over that length,
+    lo = max(floor(c(fast)), 0), hi = min(ceil(c(slow)), rope_dim - 1), r_n = clamp((n - lo) / max(hi - lo, 0.001), 0, 1),
+    the frequency is f_n / factor * r_n + f_n (1 - r_n) (slow waves are stretched by the factor, fast ones stay, those
+    between are blended), and cosines and sines are multiplied by 0.1 ln(factor) + 1. The table of frequencies is made
+    on the host in float64 and kept in float32; angles, cosines and sines are the kernel's, in float32."""
+    capturable = True
+    RAMP_FLOOR = 0.001
+    MAGNITUDE_SLOPE = 0.1
+
+    def __init__(self, rope_dim: int, base: float, neighbours: bool = True, scaling: Optional[dict] = None):
+        if rope_dim <= 0 or rope_dim % 2 != 0:
+            raise ValueError(f"rotary width must be positive and even, found {rope_dim}")
+        self.rope_dim, self.base, self.neighbours = int(rope_dim), float(base), bool(neighbours)
+        self.scaling = None if not scaling else {key: float(scaling[key]) for key in ("factor", "original", "fast", "slow")}
+        self.frequencies = None
+        self.magnitude = 1.0 if self.scaling is None else self.MAGNITUDE_SLOPE * math.log(self.scaling["factor"]) + 1.0
+
+    def frequency_table(self):
+        """The pairs' frequencies, as Python floats."""
+        plain = [self.base ** (-2.0 * n / self.rope_dim) for n in range(self.rope_dim // 2)]
+        if self.scaling is None:
+            return plain
+        c = self.scaling
+
+        def pair_of(turns: float) -> float:
+            return self.rope_dim * math.log(c["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
+
+        lo = max(math.floor(pair_of(c["fast"])), 0)
+        hi = min(math.ceil(pair_of(c["slow"])), self.rope_dim - 1)
+        out = []
+        for n, f in enumerate(plain):
+            ramp = min(max((n - lo) / max(hi - lo, self.RAMP_FLOOR), 0.0), 1.0)
+            out.append(f / c["factor"] * ramp + f * (1.0 - ramp))
+        return out
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        if self.frequencies is not None and getattr(self, "runtime", None) is runtime:
+            return
+        super().bind(tensors, runtime)
+        self.frequencies = torch.tensor(self.frequency_table(), dtype=torch.float64).to(torch.float32).to(runtime.device)
+
+    def pair_rotation(self):
+        """(frequencies float32 [rope_dim / 2] on the device, rope_dim, neighbours, magnitude): for the kernel that completes
+        q and k after their projection."""
+        return self.frequencies, self.rope_dim, self.neighbours, self.magnitude
+
+    def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch) -> None:
+        raise NotImplementedError("a rotation of pairs with a table of frequencies is done by the kernel that completes q and k")
+
+
+class DistanceBuckets(PositionEncoding):
+    """Positions enter the scores only: a learnt number per head and bucket of distance is added to the scaled score.
+    The table `name` is [rows, n_heads]; a key n tokens behind the query reads row n for n < rows / 2 (halves rounded
+    down), else row min(rows - 1, rows / 2 + floor(ln(n / (rows / 2)) / ln(far / (rows / 2)) * (rows - rows / 2))): steps
+    that grow with the distance and reach the last row at `far`. Bound, it is a dense table [n_heads, span] by distance,
+    whose last column holds for every distance beyond."""
+    capturable = True
+
+    def __init__(self, name: str, n_heads: int, rows: int, far: float):
+        if rows < 2 or far <= rows // 2:
+            raise ValueError(f"a table of {rows} buckets that ends at distance {far}: two rows at least, and an end beyond half of them")
+        self.name, self.n_heads, self.rows, self.far = name, int(n_heads), int(rows), float(far)
+        self.table = None
+
+    def weight_specs(self):
+        from .base import WeightSpec
+        return {self.name: WeightSpec((self.rows, self.n_heads), kind="vector")}
+
+    def bucket(self, n: int) -> int:
+        half = self.rows // 2
+        if n < half:
+            return n
+        return min(self.rows - 1, half + int(math.floor(math.log(n / half) / math.log(self.far / half) * (self.rows - half))))
+
+    def bind(self, tensors, runtime: Runtime) -> None:
+        super().bind(tensors, runtime)
+        span = 1
+        while self.bucket(span - 1) < self.rows - 1:
+            span += 1
+        rows = torch.tensor([self.bucket(n) for n in range(span)], dtype=torch.long)
+        learnt = tensors[self.name].to(torch.float32).to("cpu")
+        self.table = learnt[rows].t().contiguous().to(runtime.device)          # [n_heads, span]
+
+    def apply(self, qkv, n_heads, n_kv_heads, head_dim, batch) -> None:
+        return None
+
+    def score_bias_table(self):
+        return self.table
+
+
+register_part("position", "pair_rotation", PairRotation)
+register_part("position", "distance_buckets", DistanceBuckets)
 register_part("position", "distance_slopes", DistanceSlopes)
 register_part("position", "rotary", Rotary)
 register_part("position", "none", NoPosition)

@@ -124,7 +124,8 @@ def warn_of_ignored(where: str, found: Iterable[str], ignored: Iterable[str]) ->
     present = sorted(set(ignored) & set(found))
     if present:
         warnings.warn(f"{where}: {', '.join(present)} ignored: the model does not read "
-                      f"{'it' if len(present) == 1 else 'them'} (a tied head uses the embedding's table)", stacklevel=3)
+                      f"{'it' if len(present) == 1 else 'them'} (a tied head uses the embedding's table; the first of the layers "
+                      "that share their values blends nothing in)", stacklevel=3)
 
 
 class CheckpointSource:
