@@ -114,6 +114,7 @@ def distance_bucket(n, rows, far):
 # ---- the two mixers ------------------------------------------------------------------------------------------
 
 def visible(i, j, window):
+    """Whether the query at position i sees the key at position j: itself and the window - 1 tokens before it."""
     return 0 <= i - j and (window is None or i - j < window)
 
 
@@ -130,18 +131,16 @@ def gated_sigmoid_attention(h, positions, m, t, p, v_first):
         q, k = rotate_neighbours(q, positions, freqs, magnitude), rotate_neighbours(k, positions, freqs, magnitude)
     if m.get("v_mix") and v_first is not None:
         lam = t[p + "vmix"]
-        v = (1 - lam) * v + lam * v_first
+        v = (1 - lam) * v + lam * v_first.reshape(T, G, e)       # (a token's values side by side, however the heads cut them)
     window = (m.get("mask") or {}).get("size")
     out = torch.zeros(T, H, e, dtype=F)
     for a in range(T):
-        for b in range(T):
-            if not visible(positions[a], positions[b], window):
-                continue
-            raw = torch.stack([q[a, head] @ k[b, head // (H // G)] for head in range(H)]) * m["scale"]
-            mixed = t[p + "talk"] @ raw
-            weight = sigmoid(mixed + t[p + "pb"])
-            for head in range(H):
-                out[a, head] += weight[head] * v[b, head // (H // G)]
+        seen = [b for b in range(T) if visible(positions[a], positions[b], window)]
+        raw = torch.stack([k[seen, head // (H // G)] @ q[a, head] for head in range(H)]) * m["scale"]      # [H, keys]
+        mixed = t[p + "talk"] @ raw                                    # every head's score is a mix of all heads' scores
+        weight = sigmoid(mixed + t[p + "pb"][:, None])                 # no normalisation over the keys
+        for head in range(H):
+            out[a, head] = weight[head] @ v[seen, head // (H // G)]
     gate = sigmoid(h @ t[p + "g"].T)                                   # [T, H]
     out = out * gate[:, :, None]
     return out.reshape(T, H * e) @ t[p + "o"].T + t[p + "o.b"], v
@@ -156,18 +155,16 @@ def biased_softmax_attention(h, positions, m, t, p, v_first, eps):
     v = (h @ t[p + "v"].T).reshape(T, G, e)
     if m.get("v_mix") and v_first is not None:
         lam = t[p + "vmix"]
-        v = (1 - lam) * v + lam * v_first
+        v = (1 - lam) * v + lam * v_first.reshape(T, G, e)       # (a token's values side by side, however the heads cut them)
     window = (m.get("mask") or {}).get("size")
     rel = t[p + "rel"]
     out = torch.zeros(T, H, e, dtype=F)
     for head in range(H):
         for a in range(T):
             seen = [b for b in range(T) if visible(positions[a], positions[b], window)]
-            scores = torch.stack([q[a, head] @ k[b, head // (H // G)] * m["scale"]
-                                  + rel[distance_bucket(positions[a] - positions[b], rel.shape[0], m["bias_max"]), head] for b in seen])
-            weights = torch.softmax(scores, 0)
-            for w, b in zip(weights, seen):
-                out[a, head] += w * v[b, head // (H // G)]
+            bias = torch.stack([rel[distance_bucket(positions[a] - positions[b], rel.shape[0], m["bias_max"]), head] for b in seen])
+            scores = k[seen, head // (H // G)] @ q[a, head] * m["scale"] + bias
+            out[a, head] = torch.softmax(scores, 0) @ v[seen, head // (H // G)]
     return out.reshape(T, H * e) @ t[p + "o"].T, v
 
 
@@ -200,3 +197,11 @@ def forward(raw, t, tokens, keep_layers=False):
         after.append(x)
     logits = layer_norm(x, t["final.norm"], t["final.norm.b"], eps) @ t["head"].T
     return (logits, torch.stack(after)) if keep_layers else logits
+
+
+class PlainModel:
+    def __init__(self, folder):
+        self.raw, self.tensors = read_folder(folder)
+
+    def logits(self, tokens):
+        return forward(self.raw, self.tensors, list(tokens))
