@@ -24,6 +24,12 @@ measures instead the Sozopel decoder (layers of time mixing, of windowed attenti
 retention, in turn) at layer sizes of real models, beside the Llama decoder of the same width, depth, heads and
 feed-forward width: a prefill of 2048 tokens and decode steps at batch 1, 8 and 64 after 1024 tokens of context, each as
 tokens a second and ms; one JSON line with both models' numbers.
+
+    python bench.py --design ledudra [--size small|medium|large] [--layers N]
+
+the same for the Ledudra decoder (attention with sigmoid weights, mixed heads and a gate under a window of 512 keys, and
+softmax attention with head norms and biases by distance under a window of 1024, in turn, every sublayer between two
+layer norms), beside the same Llama decoder.
 """
 import argparse
 import json
@@ -119,6 +125,26 @@ def sozopel_config(size, layers, max_positions):
             "canon": {"taps": 4}, "layers": [kinds[order[i % 3]] for i in range(layers)]}
 
 
+def ledudra_config(size, layers, max_positions):
+    w, d, ff = size["width"], size["head"], size["ff"]
+    heads = w // d
+    kv_heads = max(1, heads // 4)
+    mlp = {"kind": "dense", "ff": ff}
+    kinds = [
+        {"type": "attention", "mlp": mlp,
+         "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "mask": {"size": 512}, "scale": d ** -0.5, "v_mix": True,
+                   "rot": {"dims": d // 2, "base": 500000.0, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}}},
+        {"type": "attention_2", "mlp": mlp,
+         "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": d, "vdim": d, "mask": {"size": 1024}, "scale": d ** -0.5, "v_mix": True,
+                   "bias_max": 2048, "bias_rows": 32}},
+    ]
+    return {"architecture": "Ledudra", "vocab": size["vocab"], "width": w, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "layers": [kinds[i % 2] for i in range(layers)]}
+
+
+DESIGN_CONFIGS = {"sozopel": sozopel_config, "ledudra": ledudra_config}
+
+
 def llama_config(size, layers, max_positions):
     w, d = size["width"], size["head"]
     return dict(COMMON, architectures=["LlamaForCausalLM"], vocab_size=size["vocab"], hidden_size=w, head_dim=d,
@@ -133,9 +159,9 @@ def run_design(args) -> int:
     layers = args.layers if args.layers is not None else 6
     context = DESIGN_CONTEXT
     most = max(DESIGN_BATCHES)
-    record = {"design": "sozopel", "beside": "llama", "size": args.size, **size, "layers": layers, "dtype": args.dtype,
+    record = {"design": args.design, "beside": "llama", "size": args.size, **size, "layers": layers, "dtype": args.dtype,
               "context": context, "prefill_tokens": PREFILL_TOKENS, "data": "synthetic token ids, random weights N(0, 0.02)"}
-    for name, raw in (("sozopel", sozopel_config(size, layers, 4096)), ("llama", llama_config(size, layers, 4096))):
+    for name, raw in ((args.design, DESIGN_CONFIGS[args.design](size, layers, 4096)), ("llama", llama_config(size, layers, 4096))):
         engine = Engine.random(parse_config(raw), seed=args.seed, dtype=args.dtype, max_tokens=max(most * context, PREFILL_TOKENS),
                                max_slots=most, max_context=max(context, PREFILL_TOKENS))
         bench = Bench(engine, args.seed)
@@ -302,7 +328,7 @@ def main() -> int:
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--phase", default="all", choices=["all", "decode", "prefill"],
                         help="for profiling: run only the decode steps, or only the prefill (prints a partial record)")
-    parser.add_argument("--design", default=None, choices=["sozopel"],
+    parser.add_argument("--design", default=None, choices=sorted(DESIGN_CONFIGS),
                         help="measure this design beside the Llama decoder of equal sizes instead (see the top of this file)")
     parser.add_argument("--size", default="medium", choices=sorted(DESIGN_SIZES), help="with --design: the layers' sizes")
     parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,

@@ -347,6 +347,20 @@ def test_attention_with_sigmoid_weights_mixed_heads_and_a_gate(n_heads, n_kv_hea
             assert torch.equal(got, first), f"cuts {cuts[:4]} change the bits"
 
 
+@pytest.mark.parametrize("window", [None, 100])
+def test_a_step_of_many_tokens_and_steps_of_few_give_the_same_bits(window, ops):
+    """A step of few tokens is shared out among more workgroups than one of many: the blocks' parts are added in the same order."""
+    n_heads, n_kv_heads, dim, vdim, length = 6, 2, 16, 24, 330
+    generator = torch.Generator().manual_seed(11)
+    q, k, v = (torch.randn(length, n * size, generator=generator) for n, size in ((n_heads, dim), (n_kv_heads, dim), (n_kv_heads, vdim)))
+    options = dict(head_mix=torch.eye(n_heads) + 0.2 * torch.randn(n_heads, n_heads, generator=generator), head_bias=torch.full((n_heads,), -2.0))
+    want = plain_weights_summed(q, k, v, n_heads, n_kv_heads, dim, vdim, 0.2, window, options["head_mix"], options["head_bias"], None)
+    whole = attend(ops, q, k, v, [length], torch.float32, n_heads, n_kv_heads, dim, vdim, 0.2, window=window, sigmoid=options)
+    assert float((whole - want).abs().max()) <= 1e-5 * float(want.abs().max())
+    for cuts in ([300, 30], [64] * 5 + [10], [290] + [1] * 40):
+        assert torch.equal(attend(ops, q, k, v, cuts, torch.float32, n_heads, n_kv_heads, dim, vdim, 0.2, window=window, sigmoid=options), whole), cuts
+
+
 @pytest.mark.parametrize("window", [1, 3, 17, 64, 70, 129])
 def test_a_key_just_inside_the_window_is_seen_and_one_just_outside_is_not(window, ops):
     """One key whose weight is one where all others' are nothing, at the last place the window keeps and at the first it

@@ -15,10 +15,51 @@ namespace {
 
 constexpr int NORM_THREADS = 256;
 
-// buf[c] = layer norm of row[c] (+ add[c]) for this thread's columns c = threadIdx.x, + 256, ...
+template <typename TW>
+__device__ __forceinline__ float4 four(const TW* __restrict__ p) {     // four elements from a place that is a multiple of four
+    if constexpr (sizeof(TW) == 4) {
+        return *reinterpret_cast<const float4*>(p);
+    } else {
+        struct alignas(8) Four { TW e[4]; };
+        const Four v = *reinterpret_cast<const Four*>(p);
+        return make_float4(to_float(v.e[0]), to_float(v.e[1]), to_float(v.e[2]), to_float(v.e[3]));
+    }
+}
+
+// buf[c] = layer norm of row[c] (+ add[c]) for this thread's columns: c = threadIdx.x, + 256, ..., or, where the row's
+// length is a multiple of four, the quads 4 threadIdx.x, + 1024, ... (the sums a thread keeps are over other columns then,
+// but which of the two it is depends on the row's length alone).
 template <typename TW>
 __device__ __forceinline__ void normalise(const float* __restrict__ row, const TW* __restrict__ add, const TW* __restrict__ w,
                                           const TW* __restrict__ b, float eps, int hidden, float* buf, float* scratch) {
+    if (hidden % 4 == 0) {
+        const int quads = hidden / 4;
+        float4* buf4 = reinterpret_cast<float4*>(buf);
+        float sum = 0.f;
+        for (int q = threadIdx.x; q < quads; q += NORM_THREADS) {
+            float4 v = *reinterpret_cast<const float4*>(row + 4 * q);
+            if (add) {
+                const float4 a = four(add + 4 * q);
+                v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+            }
+            buf4[q] = v;
+            sum += (v.x + v.y) + (v.z + v.w);
+        }
+        const float mean = block_sum(sum, scratch) / (float)hidden;
+        float squares = 0.f;
+        for (int q = threadIdx.x; q < quads; q += NORM_THREADS) {
+            const float4 v = buf4[q];
+            const float dx = v.x - mean, dy = v.y - mean, dz = v.z - mean, dw = v.w - mean;
+            squares = fmaf(dx, dx, fmaf(dy, dy, fmaf(dz, dz, fmaf(dw, dw, squares))));
+        }
+        const float inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)hidden + eps);
+        for (int q = threadIdx.x; q < quads; q += NORM_THREADS) {
+            const float4 v = buf4[q], g = four(w + 4 * q), s = four(b + 4 * q);
+            buf4[q] = make_float4(fmaf((v.x - mean) * inv, g.x, s.x), fmaf((v.y - mean) * inv, g.y, s.y),
+                                  fmaf((v.z - mean) * inv, g.z, s.z), fmaf((v.w - mean) * inv, g.w, s.w));
+        }
+        return;
+    }
     float sum = 0.f;
     for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) {
         const float v = row[c] + (add ? to_float(add[c]) : 0.f);
@@ -35,15 +76,28 @@ __device__ __forceinline__ void normalise(const float* __restrict__ row, const T
     for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) buf[c] = fmaf((buf[c] - mean) * inv, to_float(w[c]), to_float(b[c]));
 }
 
+// Every thread's columns of a row, as `normalise` deals them: body(c) for each.
+template <typename Body>
+__device__ __forceinline__ void for_my_columns(int hidden, Body body) {
+    if (hidden % 4 == 0) {
+        for (int q = threadIdx.x; q < hidden / 4; q += NORM_THREADS) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) body(4 * q + e);
+        }
+    } else {
+        for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) body(c);
+    }
+}
+
 template <typename TW, typename TO>
 __global__ void __launch_bounds__(NORM_THREADS) layernorm_kernel(const float* __restrict__ x, const TW* __restrict__ w, const TW* __restrict__ b,
                                                                  float eps, TO* __restrict__ out, const int* __restrict__ rows, int hidden) {
-    extern __shared__ float buf[];
+    extern __shared__ __attribute__((aligned(16))) float buf[];
     __shared__ float scratch[32];
     const long src = rows ? rows[blockIdx.x] : blockIdx.x;
     normalise<TW>(x + src * hidden, nullptr, w, b, eps, hidden, buf, scratch);
     TO* dst = out + (long)blockIdx.x * hidden;
-    for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) dst[c] = from_float<TO>(buf[c]);
+    for_my_columns(hidden, [&](int c) { dst[c] = from_float<TO>(buf[c]); });
 }
 
 // Row r is a token of the sequence in token_slots[r] (negative: padding, zeros out). The token before it is row r - 1 if that
@@ -54,7 +108,7 @@ __global__ void __launch_bounds__(NORM_THREADS) layernorm_shift_kernel(const flo
                                                                        const TW* __restrict__ mix, float eps, float* __restrict__ state,
                                                                        const int* __restrict__ token_slots, TO* __restrict__ out, int hidden,
                                                                        int with_state) {
-    extern __shared__ float buf[];                             // [2][hidden]: this row's norm, the one before
+    extern __shared__ __attribute__((aligned(16))) float buf[];                             // [2][hidden]: this row's norm, the one before
     __shared__ float scratch[32];
     const long r = blockIdx.x;
     const int slot = token_slots[r];
@@ -71,13 +125,13 @@ __global__ void __launch_bounds__(NORM_THREADS) layernorm_shift_kernel(const flo
     if (in_step) {
         normalise<TW>(x + (r - 1) * hidden, nullptr, w, b, eps, hidden, before, scratch);
     } else {
-        for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) before[c] = kept[c];
+        for_my_columns(hidden, [&](int c) { before[c] = kept[c]; });
     }
-    for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) {
+    for_my_columns(hidden, [&](int c) {
         const float h = here[c];
         dst[c] = from_float<TO>(fmaf(before[c] - h, to_float(mix[c]), h));
         if (with_state) kept[c] = h;
-    }
+    });
 }
 
 // The state after a step of several tokens a sequence: the norm of each sequence's last row (a launch of its own, after
@@ -86,14 +140,14 @@ template <typename TW>
 __global__ void __launch_bounds__(NORM_THREADS) layernorm_state_kernel(const float* __restrict__ x, const TW* __restrict__ w, const TW* __restrict__ b,
                                                                        float eps, float* __restrict__ state, const int* __restrict__ seq_offsets,
                                                                        const int* __restrict__ seq_slots, int hidden) {
-    extern __shared__ float buf[];
+    extern __shared__ __attribute__((aligned(16))) float buf[];
     __shared__ float scratch[32];
     const int seq = blockIdx.x, slot = seq_slots[seq];
     const int begin = seq_offsets[seq], end = seq_offsets[seq + 1];
     if (slot < 0 || end <= begin) return;
     normalise<TW>(x + (long)(end - 1) * hidden, nullptr, w, b, eps, hidden, buf, scratch);
     float* kept = state + (long)slot * hidden;
-    for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) kept[c] = buf[c];
+    for_my_columns(hidden, [&](int c) { kept[c] = buf[c]; });
 }
 
 template <typename TW, typename TO>
@@ -102,17 +156,17 @@ __global__ void __launch_bounds__(NORM_THREADS) add_layernormed_kernel(float* __
                                                                        const TW* __restrict__ b, float eps, float scale,
                                                                        const TW* __restrict__ next_w, const TW* __restrict__ next_b, float next_eps,
                                                                        TO* __restrict__ next_out, int hidden) {
-    extern __shared__ float buf[];
+    extern __shared__ __attribute__((aligned(16))) float buf[];
     __shared__ float scratch[32];
     const long r = blockIdx.x;
     normalise<TW>(y + r * hidden, pre_bias, w, b, eps, hidden, buf, scratch);
     float* row = residual + r * hidden;
-    for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) row[c] = fmaf(scale, buf[c], row[c]);
+    for_my_columns(hidden, [&](int c) { row[c] = fmaf(scale, buf[c], row[c]); });
     if (next_out == nullptr) return;
     // (every thread reads back the columns it has just written itself)
     normalise<TW>(row, nullptr, next_w, next_b, next_eps, hidden, buf, scratch);
     TO* dst = next_out + r * hidden;
-    for (int c = threadIdx.x; c < hidden; c += NORM_THREADS) dst[c] = from_float<TO>(buf[c]);
+    for_my_columns(hidden, [&](int c) { dst[c] = from_float<TO>(buf[c]); });
 }
 
 bool known(int dtype) { return dtype == XRT_F32 || dtype == XRT_BF16; }

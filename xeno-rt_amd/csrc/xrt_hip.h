@@ -269,11 +269,16 @@ int xrt_attention_general(const void* qkv, int dtype, int tokens, int n_heads, i
 // before that the heads' scaled scores of a (query, key) pair are mixed, score_h <- sum_g head_mix[h][g] score_g
 // (head_mix float32 [n_heads][n_heads], or null); a head's summed values are multiplied by sigmoid(gate[token][h]) (float32
 // rows gate_stride apart, or null). q: rows of n_heads x head_dim, q_stride apart; out rows n_heads x value_dim; keys and
-// values come from the cache (the step's own included, which must have been written). window 0: none.
+// values come from the cache (the step's own included, which must have been written). window 0: none. A step of few tokens
+// runs faster shared out among more workgroups, through a workspace of xrt_attention_sigmoid_workspace(...) floats (0:
+// not needed; max_context: the longest sequence after the step, 0 if unknown); without it the step runs a workgroup a
+// token, to the same bits.
+long xrt_attention_sigmoid_workspace(long tokens, int n_heads, int head_dim, int value_dim, int window, int max_context);
 int xrt_attention_sigmoid(const void* q, long q_stride, int dtype, long tokens, int n_heads, int n_kv_heads, int head_dim,
                           int value_dim, const void* k_cache, const void* v_cache, const int* block_table, int table_stride,
                           int n_blocks, const int* positions, const int* slots, void* out, float scale, int window,
-                          const float* head_mix, const float* head_bias, const float* gate, long gate_stride, void* stream);
+                          const float* head_mix, const float* head_bias, const float* gate, long gate_stride,
+                          int max_context, float* workspace, long workspace_floats, void* stream);
 
 // Between an attention's projection (float32 sums, rows [q heads | k heads | v heads | anything], proj_stride apart) and its
 // scores: biases ([heads * dim] each, or null); an RMS norm of every head of q and k with one weight [head_dim] each (or

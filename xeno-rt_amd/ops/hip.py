@@ -194,6 +194,7 @@ class HipOps:
         self.lib.xrt_probe_read_bytes.restype = ctypes.c_long
         self.lib.xrt_sample_workspace.restype = ctypes.c_long
         self.lib.xrt_linear_recurrence_workspace.restype = ctypes.c_long
+        self.lib.xrt_attention_sigmoid_workspace.restype = ctypes.c_long
 
     # -- helpers -------------------------------------------------------------
     def _check(self, status: int) -> None:
@@ -543,6 +544,7 @@ class HipOps:
         head_mix: float32 [n_heads, n_heads], the heads' scaled scores of a (query, key) pair are multiplied by it before the
         sigmoid; head_bias: float32 [n_heads]; gate: float32 rows with one number per head (columns of a wider matrix, if
         need be): a head's output is multiplied by sigmoid(gate)."""
+        from ..cache import BLOCK_TOKENS
         tokens = q.shape[0]
         q_stride = self._rows(q, "attention q", n_heads * head_dim)
         self._require(out, "attention out", q.dtype, (tokens, n_heads * value_dim), q)
@@ -554,10 +556,17 @@ class HipOps:
         if head_bias is not None:
             self._require(head_bias, "attention head_bias", torch.float32, (n_heads,), q)
         gate_stride = 0 if gate is None else self._rows(gate, "attention gate", n_heads, torch.float32, q)
+        # a step of few tokens is shared out among more workgroups, if the batch says how long its sequences are
+        max_context = int(getattr(batch, "max_context", 0) or 0)
+        if max_context > stride * BLOCK_TOKENS:
+            raise KernelError(f"attention: a sequence of {max_context} tokens exceeds the block table")
+        need = int(self.lib.xrt_attention_sigmoid_workspace(ctypes.c_long(tokens), n_heads, head_dim, value_dim, int(window or 0), max_context))
+        workspace = self._empty(need, torch.float32, q.device) if need > 0 else None
         self._check(self.lib.xrt_attention_sigmoid(
             _ptr(q), ctypes.c_long(q_stride), _code(q), ctypes.c_long(tokens), n_heads, n_kv_heads, head_dim, value_dim, _ptr(k_cache),
             _ptr(v_cache), _ptr(table), stride, n_blocks, _ptr(batch.positions), _ptr(batch.slots), _ptr(out), ctypes.c_float(scale),
-            int(window or 0), _ptr(head_mix), _ptr(head_bias), _ptr(gate), ctypes.c_long(gate_stride), self._stream(q)))
+            int(window or 0), _ptr(head_mix), _ptr(head_bias), _ptr(gate), ctypes.c_long(gate_stride), max_context, _ptr(workspace),
+            ctypes.c_long(need), self._stream(q)))
 
     def qkv_complete(self, proj, n_heads, n_kv_heads, head_dim, value_dim, batch, q_out, kv=None, biases=None, norms=None,
                      norm_eps=0.0, frequencies=None, rot_dims=0, neighbours=True, magnitude=1.0, values_in=None, values_out=None,
