@@ -328,7 +328,8 @@ def plain_weights_summed(q, k, v, n_heads, n_kv_heads, dim, vdim, scale, window,
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n_heads,n_kv_heads,dim,vdim,window", [(6, 3, 20, 12, 17), (2, 2, 32, 32, 70), (8, 1, 16, 8, 3), (1, 1, 64, 96, None),
-                                                               (12, 2, 48, 20, 64), (3, 1, 7, 130, 129), (5, 5, 136, 9, 65)])
+                                                               (12, 2, 48, 20, 64), (3, 1, 7, 130, 129), (5, 5, 136, 9, 65),
+                                                               (32, 8, 128, 128, 100)])         # (the last: more LDS than a launch has by default)
 def test_attention_with_sigmoid_weights_mixed_heads_and_a_gate(n_heads, n_kv_heads, dim, vdim, window, dtype, ops):
     length = 150
     generator = torch.Generator().manual_seed(dim + vdim)
@@ -574,13 +575,13 @@ def random_configuration(seed):
         if kind == "attention":
             if r.random() < 0.8:
                 dims = r.choice([d for d in (2, 4, 6, 16, 20, 32, 64) if d <= mixer["dim"]])
-                mixer["rot"] = {"dims": dims, "base": r.choice([100.0, 10000.0, 250000.0])}
+                mixer["rot"] = {"dims": dims, "base": r.choice([100.0, 10000.0, 1000000.0])}
                 if r.random() < 0.6:
                     mixer["rot"]["scaling"] = {"factor": r.choice([2.0, 4.0, 16.0]), "original": r.choice([16, 64, 256]),
                                                "fast": r.choice([8.0, 32.0]), "slow": r.choice([0.5, 1.0, 2.0])}
         else:
             mixer["bias_rows"] = r.choice([2, 5, 8, 16, 33])
-            mixer["bias_max"] = r.choice([n for n in (3, 20, 64, 120, 500) if n > mixer["bias_rows"] // 2])
+            mixer["bias_max"] = r.choice([n for n in (3, 20, 64, 150, 500) if n > mixer["bias_rows"] // 2])
         layers.append({"type": kind, "mixer": mixer, "mlp": r.choice([None, {"kind": "dense", "ff": r.choice([16, 56, 104])}])})
     return {"architecture": "Ledudra", "vocab": r.choice([50, 97, 160]), "width": width, "norm": {"eps": r.choice([1e-6, 1e-5, 1e-3])},
             "residual_mult": r.choice([0.3, 1.0, 2.0]), "layers": layers}

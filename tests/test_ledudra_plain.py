@@ -48,15 +48,15 @@ def test_stretched_frequencies():
 
 
 def test_buckets_of_distance():
-    rows, far = 16, 120
-    assert [P.distance_bucket(n, rows, far) for n in range(8)] == list(range(8))       # below half the rows: the distance itself
-    assert P.distance_bucket(8, rows, far) == 8 and P.distance_bucket(119, rows, far) == 15 and P.distance_bucket(10 ** 6, rows, far) == 15
+    rows, far = 12, 90
+    assert [P.distance_bucket(n, rows, far) for n in range(6)] == list(range(6))       # below half the rows: the distance itself
+    assert P.distance_bucket(6, rows, far) == 6 and P.distance_bucket(89, rows, far) == 11 and P.distance_bucket(10 ** 6, rows, far) == 11
     buckets = [P.distance_bucket(n, rows, far) for n in range(200)]
-    assert buckets == sorted(buckets) and set(buckets) == set(range(16))
-    # a step of the logarithm: 8 * 15^(k / 8) is where bucket 8 + k begins
-    for k in range(1, 8):
-        edge = 8 * 15 ** (k / 8)
-        assert P.distance_bucket(math.ceil(edge), rows, far) == 8 + k and P.distance_bucket(math.ceil(edge) - 1, rows, far) == 8 + k - 1
+    assert buckets == sorted(buckets) and set(buckets) == set(range(12))
+    # a step of the logarithm: 6 * 15^(k / 6) is where bucket 6 + k begins
+    for k in range(1, 6):
+        edge = 6 * 15 ** (k / 6)
+        assert P.distance_bucket(math.ceil(edge), rows, far) == 6 + k and P.distance_bucket(math.ceil(edge) - 1, rows, far) == 6 + k - 1
     assert [P.distance_bucket(n, 7, 20) for n in (2, 3, 4, 19, 20)] == [2, 3, 3, 6, 6]   # an odd number of rows: half is 3, four rows beyond
 
 
