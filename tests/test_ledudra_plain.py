@@ -141,3 +141,19 @@ def test_the_model_declares_the_designs_tensors():
     assert [need.kv.window for need in needs] == [17, 70, None] and [need.kv.value_width for need in needs] == [12, 36, 18]
     assert all(dict(need.states)["shift"].shape == (1, 40) for need in needs)
     assert spec.capturable()
+
+
+def test_a_layer_that_shares_no_values_may_still_carry_its_share():
+    """A checkpoint may hold the share of a blend for a layer that blends nothing in: the model lists it as not read."""
+    import copy
+    from xeno_rt_amd.config import architecture, parse_config
+    from xeno_rt_amd.weights.loader import check_names
+    raw = copy.deepcopy(CONFIGS["wide"])
+    raw["layers"][3]["mixer"].pop("v_mix")                              # (absent means no)
+    spec = architecture("Ledudra").build(parse_config(raw))
+    assert sorted(spec.ignored_names()) == ["l2.mix.vmix", "l3.mix.vmix"]
+    names = spec.weight_specs()
+    assert "l0.mix.vmix" in names and "l1.mix.vmix" in names and "l2.mix.vmix" not in names
+    found = {name: ("BF16", tuple(s.shape)) for name, s in names.items()}
+    found["l3.mix.vmix"] = ("BF16", ())
+    check_names("a folder", names, found, spec.ignored_names())
